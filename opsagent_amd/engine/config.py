@@ -199,7 +199,10 @@ class MixerSpec:
     """One layer's token mixer. kind: "attention" (distance-penalty softmax
     attention) | "channel_delta" (gated delta rule) | "rotary_window"
     (rotary softmax attention with per-head query/key norm, an optional
-    sliding window and an optional sink term)."""
+    sliding window and an optional sink term) | "latent_attention" (softmax
+    attention over a cached low-rank latent and one rotated key part shared
+    by the heads) | "lightning" (linear attention with one fixed decay per
+    head) | "gla" (linear attention with a learned decay per key channel)."""
 
     kind: str
     heads: int
@@ -221,14 +224,25 @@ class MixerSpec:
     window: Optional[int] = None
     # a learned per-head term in the softmax denominator
     sink: bool = False
+    # latent attention: size of the cached latent, rotated channels per head
+    # (query) and of the shared key part, and the layer whose cached latent
+    # this layer reads instead of projecting its own (None = its own)
+    kv_rank: int = 0
+    rot_dim: int = 0
+    kv_from: Optional[int] = None
+    # linear attention: fixed per-head decays ("lightning"), temperature of
+    # the learned per-channel decay sigmoid(z)^(1/tau) ("gla")
+    decay: Optional[List[float]] = None
+    tau: float = 1.0
 
     @property
     def has_kv(self) -> bool:
-        return self.kind in ("attention", "rotary_window")
+        return self.kind in ("attention", "rotary_window") or (
+            self.kind == "latent_attention" and self.kv_from is None)
 
     @property
     def has_state(self) -> bool:
-        return self.kind == "channel_delta"
+        return self.kind in ("channel_delta", "lightning", "gla")
 
 
 @dataclasses.dataclass
@@ -237,8 +251,14 @@ class RouterSpec:
     logits become scores s ("sigmoid" | "softmax"); with `correction` the
     ranking uses c = s + a learned vector while the mixing weights keep s;
     `groups` > 1 cuts the experts into runs of neighbours rated
-    max1(c) + max2(c), of which the `keep` top-rated may be picked from;
-    w_j = scale * s_j / sum_k s_k over the `top` picked experts."""
+    max1(c) + max2(c) (`rating` "top2") or max(c) ("max"), of which the
+    `keep` top-rated may be picked from; w_j = scale * s_j / sum_k s_k over
+    the `top` picked experts, or scale * s_j with renorm=False.
+    act: the experts' gate activation ("silu" | "gelu_tanh" | "clamp_swish":
+    g = min(gate, limit), u = clamp(up, -limit, limit),
+    y = g sigmoid(alpha g) (u + 1)); the shared expert has its own limit and,
+    with shared_gate, is scaled per token by the sigmoid of a learned
+    projection."""
 
     experts: int
     top: int
@@ -249,6 +269,13 @@ class RouterSpec:
     keep: int = 1
     scale: float = 1.0
     shared_ff: int = 0               # inner size of the always-on expert (0 = none)
+    rating: str = "top2"
+    renorm: bool = True
+    act: str = "silu"
+    limit: float = 0.0
+    alpha: float = 1.702
+    shared_limit: float = 0.0
+    shared_gate: bool = False
 
 
 @dataclasses.dataclass
@@ -275,8 +302,9 @@ class HybridSpec:
     logit_softcap: Optional[float] = None
     # "post_canon": grouped RMS norm on sublayer outputs, sublayers read
     # x + canon(x). "sandwich": a dynamic-tanh norm before and after every
-    # sublayer.
+    # sublayer. "pre_norm": a weighted layer norm before every sublayer.
     layer_style: str = "post_canon"
+    embed_scale: float = 1.0
     max_seq_len: int = 1 << 20
     weights_path: Optional[str] = None
 
@@ -454,9 +482,139 @@ def vazilorn_config_dict(
             "vocab": vocab, "width": width}
 
 
+def rafodra_spec_from_dict(cfg: dict, name: str = "rafodra") -> HybridSpec:
+    """Parse a Rafodra config.json dict: pre-norm layers whose mixer is
+    latent attention (optionally reading another layer's cached latent),
+    lightning attention or gated linear attention, with dense silu or routed
+    clamped-swish feed-forwards."""
+    layers = []
+    for i, entry in enumerate(cfg["layers"]):
+        kind, m = entry["type"], entry["mixer"]
+        if kind == "latent_attention":
+            rot = m.get("rot") or {}
+            src = m.get("kv_from")
+            mixer = MixerSpec(
+                kind=kind, heads=int(m["heads"]), kv_heads=1, dim=int(m["dim"]),
+                vdim=int(m["vdim"]), scale=float(m["scale"]) if "scale" in m else None,
+                rot_dims=int(rot.get("dims", m["rot_dim"])),
+                rot_base=float(rot.get("base", 10000.0)),
+                kv_rank=int(m["kv_rank"]), rot_dim=int(m["rot_dim"]),
+                kv_from=None if src is None else int(src), sink=True,
+            )
+            if mixer.rot_dims % 2 or mixer.rot_dims > mixer.rot_dim:
+                raise ValueError("rot.dims must be even and at most rot_dim")
+            if mixer.kv_from is not None:
+                j = mixer.kv_from
+                if not 0 <= j < i or layers[j].mixer.kind != kind or layers[j].mixer.kv_from is not None:
+                    raise ValueError(f"layer {i}: kv_from must name an earlier latent-attention "
+                                     "layer that projects its own latent")
+                o = layers[j].mixer
+                if (o.kv_rank, o.rot_dim, o.rot_dims, o.rot_base) != (
+                        mixer.kv_rank, mixer.rot_dim, mixer.rot_dims, mixer.rot_base):
+                    raise ValueError(f"layer {i}: latent sizes differ from layer {j}'s")
+        elif kind == "lightning":
+            mixer = MixerSpec(kind=kind, heads=int(m["heads"]), kv_heads=int(m["heads"]),
+                              dim=int(m["dim"]), vdim=int(m["vdim"]),
+                              decay=[float(d) for d in m["decay"]])
+            if len(mixer.decay) != mixer.heads:
+                raise ValueError("lightning: one decay per head")
+        elif kind == "gla":
+            mixer = MixerSpec(kind=kind, heads=int(m["heads"]), kv_heads=int(m["heads"]),
+                              dim=int(m["dim"]), vdim=int(m["vdim"]), tau=float(m["tau"]))
+        else:
+            raise ValueError(f"unknown Rafodra layer type {kind!r}")
+        mlp = entry.get("mlp")
+        ls = HybridLayerSpec(mixer=mixer)
+        if mlp is not None:
+            mk = mlp.get("kind")
+            if mk == "dense":
+                ls.mlp_kind, ls.mlp_ff, ls.mlp_act = "dense", int(mlp["ff"]), "silu"
+            elif mk == "moe":
+                r = mlp["router"]
+                grp = r.get("groups") or {}
+                shared = mlp.get("shared") or {}
+                ls.mlp_kind = "moe"
+                ls.router = RouterSpec(
+                    experts=int(r["experts"]), top=int(r["top"]), ff=int(mlp["expert"]["ff"]),
+                    score="softmax", correction=False, groups=int(grp.get("count", 1)),
+                    keep=int(grp.get("keep", grp.get("count", 1))),
+                    scale=float(r.get("scale", 1.0)), shared_ff=int(shared.get("ff", 0)),
+                    rating="max", renorm=False, act="clamp_swish",
+                    limit=float(mlp["expert"]["limit"]),
+                    shared_limit=float(shared.get("limit", 0.0)), shared_gate=bool(shared),
+                )
+                if ls.router.experts % ls.router.groups:
+                    raise ValueError("experts must be a multiple of groups.count")
+            else:
+                raise ValueError(f"unknown Rafodra feed-forward kind {mk!r}")
+        layers.append(ls)
+    return HybridSpec(
+        name=name, architecture="Rafodra", vocab_size=int(cfg["vocab"]),
+        hidden_size=int(cfg["width"]), layers=layers, norm_eps=float(cfg["norm"]["eps"]),
+        layer_style="pre_norm", embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)),
+    )
+
+
+def rafodra_config_dict(
+    vocab: int, width: int, pattern: str, heads: int = 4, dim: int = 16, vdim: int = 16,
+    ff: int = 128, kv_rank: int = 24, rot_dim: int = 8, rot_base: float = 10000.0,
+    scale: Optional[float] = None, lin_heads: Optional[int] = None, lin_dim: Optional[int] = None,
+    lin_vdim: Optional[int] = None, decay: Optional[List[float]] = None, tau: float = 16.0,
+    experts: int = 8, top: int = 2, expert_ff: int = 32, groups: int = 2, keep: int = 1,
+    router_scale: float = 1.0, limit: float = 1.5, shared_ff: int = 0, shared_limit: float = 2.0,
+    embed_scale: float = 1.0, eps: float = 1e-6,
+) -> dict:
+    """A Rafodra config.json dict from a layer pattern, one or two characters
+    per layer: the mixer 'A' (latent attention), 'S' (latent attention
+    reading the latest 'A' layer's latent), 'L' (lightning), 'G' (gla),
+    followed by the feed-forward 'd' (dense), 'm' (routed experts) or '-'
+    (none)."""
+    if len(pattern) % 2:
+        raise ValueError("pattern: two characters per layer")
+    lh, ld, lv = lin_heads or heads, lin_dim or dim, lin_vdim or vdim
+    if decay is None:
+        decay = [1.0 - 2.0 ** (-(2 + 2 * h)) for h in range(lh)]
+    layers, last_a = [], None
+    for i in range(0, len(pattern), 2):
+        mk, fk = pattern[i], pattern[i + 1]
+        if mk in "AS":
+            mixer = {"heads": heads, "dim": dim, "vdim": vdim, "kv_rank": kv_rank,
+                     "rot_dim": rot_dim, "rot": {"base": rot_base, "dims": rot_dim},
+                     "scale": scale if scale is not None else (dim + rot_dim) ** -0.5}
+            if mk == "S":
+                if last_a is None:
+                    raise ValueError("'S' needs an earlier 'A' layer")
+                mixer["kv_from"] = last_a
+            else:
+                last_a = len(layers)
+            kind = "latent_attention"
+        elif mk == "L":
+            mixer, kind = {"heads": lh, "dim": ld, "vdim": lv, "decay": list(decay)}, "lightning"
+        elif mk == "G":
+            mixer, kind = {"heads": lh, "dim": ld, "vdim": lv, "tau": tau}, "gla"
+        else:
+            raise ValueError(f"unknown mixer letter {mk!r}")
+        if fk == "d":
+            mlp = {"kind": "dense", "ff": ff}
+        elif fk == "m":
+            mlp = {"kind": "moe", "expert": {"ff": expert_ff, "limit": limit},
+                   "router": {"experts": experts, "top": top, "scale": router_scale,
+                              "groups": {"count": groups, "keep": keep}}}
+            if shared_ff:
+                mlp["shared"] = {"ff": shared_ff, "limit": shared_limit}
+        elif fk == "-":
+            mlp = None
+        else:
+            raise ValueError(f"unknown feed-forward letter {fk!r}")
+        layers.append({"type": kind, "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Rafodra", "embedding": {"scale": embed_scale}, "layers": layers,
+            "norm": {"eps": eps}, "vocab": vocab, "width": width}
+
+
 # config.json "architecture" -> parser
 ARCHITECTURE_PARSERS = {"Povazen": povazen_spec_from_dict,
-                        "Vazilorn": vazilorn_spec_from_dict}
+                        "Vazilorn": vazilorn_spec_from_dict,
+                        "Rafodra": rafodra_spec_from_dict}
 
 # named hybrid configurations (random-weight benchmarking and tests)
 HYBRID_REGISTRY = {
@@ -492,6 +650,24 @@ HYBRID_REGISTRY = {
     "vazilorn-4l2k": lambda: vazilorn_config_dict(
         vocab=2048, width=2048, pattern="dddd", heads=16, kv_heads=4, dim=128,
         vdim=128, ff=8192, window=1024),
+    # CPU-test size: every mixer and feed-forward kind once
+    "rafodra-tiny": lambda: rafodra_config_dict(
+        vocab=512, width=64, pattern="LdGmAdSmL-", heads=4, dim=16, vdim=8, ff=128,
+        kv_rank=24, rot_dim=8, lin_heads=2, lin_dim=16, lin_vdim=24, experts=8, top=2,
+        expert_ff=32, groups=2, keep=1, router_scale=1.5, shared_ff=48, embed_scale=4.0),
+    # GPU-smoke size
+    "rafodra-micro": lambda: rafodra_config_dict(
+        vocab=2048, width=1024, pattern="LdGmAdLmSd", heads=8, dim=64, vdim=64, ff=2816,
+        kv_rank=128, rot_dim=32, lin_heads=8, lin_dim=128, lin_vdim=128, experts=16, top=4,
+        expert_ff=512, groups=4, keep=2, router_scale=2.0, shared_ff=512, embed_scale=8.0),
+    # layer shapes of ~1B- and ~8B-class models at 4 layers (speed beside
+    # Povazen and llama layers of equal width)
+    "rafodra-4l2k": lambda: rafodra_config_dict(
+        vocab=2048, width=2048, pattern="LdGdAdSd", heads=16, dim=128, vdim=128, ff=8192,
+        kv_rank=192, rot_dim=64, lin_heads=16, lin_dim=128, lin_vdim=128),
+    "rafodra-4l4k": lambda: rafodra_config_dict(
+        vocab=2048, width=4096, pattern="LdGdAdSd", heads=32, dim=128, vdim=128, ff=14336,
+        kv_rank=192, rot_dim=64, lin_heads=32, lin_dim=128, lin_vdim=128),
 }
 
 

@@ -366,7 +366,8 @@ class LLMEngine:
         if self.hybrid:
             esz = 4 if self.dtype == torch.float32 else 2
             per_token = sum(
-                sh[0] * (sh[1] + sh[2]) for sh in self.model.kv_layer_shapes() if sh
+                sh[0] * (sh[1] + (0 if len(sh) > 3 else sh[2]))
+                for sh in self.model.kv_layer_shapes() if sh
             )
             block_bytes = max(1, per_token * self.block_size * esz)
         else:

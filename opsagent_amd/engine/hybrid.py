@@ -14,8 +14,16 @@ Layer:  x <- x + post1(mixer(pre1(x)));  x <- x + post2(ff(pre2(x))),
 every norm elementwise: tanh(a x) w + b with one scalar a, no statistics
 over channels.
 
+"pre_norm" (the Rafodra design): latent attention (a cached low-rank latent
+and one rotated key part shared by the heads, optionally read from another
+layer's cache), lightning attention (fixed per-head decay) or gated linear
+attention (learned per-channel decay); dense silu or routed clamped-swish
+feed-forwards.
+Layer:  x <- x + mixer(ln1(x));  x <- x + ff(ln2(x)),
+ln a layer norm with a weight and no bias.
+
 The mixers are modules of their own (BiasedAttentionMixer,
-ChannelDeltaMixer) with every constant a constructor argument, built on the
+ChannelDeltaMixer, ...) with every constant a constructor argument, built on the
 flat multi-sequence ops of opsagent_amd.ops.mixer_ops; the model keeps no
 cache and no loop of its own — keys/values live in the engine's paged cache,
 recurrent and convolution state in its StateSlotPool, and one forward serves
@@ -215,12 +223,189 @@ class ChannelDeltaMixer(nn.Module):
         return ops.linear(y, self.o_w)
 
 
+class LatentAttentionMixer(nn.Module):
+    """Causal softmax attention whose keys and values are up-projections of
+    one cached latent per token. With h the input, per token the cache row
+    is [c | r]: c = rms_norm(first kv_rank rows of W_dkv h) (weighted), r =
+    the last rot_dim rows rotated by position (one key part for all heads).
+    Head h's score is (qu_h . W_uk,h c + qr_h . r) * scale with qu_h the
+    `dim` unrotated and qr_h the rot_dim rotated channels of its query; its
+    value is W_uv,h c. Because both up-projections are linear they are taken
+    to the query side: qu_h^T W_uk,h is a query against c itself, the
+    softmax weights average c, and W_uv,h is applied to that average. The
+    attention kernel therefore sees ONE key/value head of size kv_rank +
+    rot_dim whose values are the first kv_rank key channels, and the cache
+    holds nothing else. The softmax normaliser also holds exp(sink_h); each
+    head's output is scaled by sigmoid(W_g h)_h.
+
+    A layer with kv_from = j projects no latent: it reads layer j's cache
+    rows with its own queries, up-projections, sinks and gates.
+
+    Fused projection rows: q | dkv (own latent only) | gate."""
+
+    def __init__(self, hidden: int, m: MixerSpec, eps: float, dtype, gen):
+        super().__init__()
+        self.H, self.D, self.Dv = m.heads, m.dim, m.vdim
+        self.R, self.rot = m.kv_rank, m.rot_dim
+        self.kv_source = m.kv_from
+        self.own = m.kv_from is None
+        self.eps = eps
+        self.scale = float(m.scale) if m.scale is not None else (m.dim + m.rot_dim) ** -0.5
+        H, D, Dv, R, rot = self.H, self.D, self.Dv, self.R, self.rot
+        dev = gen.device
+        self.n_q = H * (D + rot)
+        self.n_kv = R + rot if self.own else 0
+        std = 1.0 / math.sqrt(hidden)
+        self.proj_w = _param(_rand(gen, self.n_q + self.n_kv + H, hidden, std=std, dtype=dtype))
+        if self.own:
+            self.dkv_norm_w = _param(1.0 + 0.1 * _rand(gen, R))
+        # up-projections per head: uk [H, D, R] (W_uk,h as stored), uv [H, Dv, R]
+        self.uk_w = _param(_rand(gen, H, D, R, std=1.0 / math.sqrt(R), dtype=dtype))
+        self.uv_w = _param(_rand(gen, H, Dv, R, std=1.0 / math.sqrt(R), dtype=dtype))
+        self.sinks = _param(_rand(gen, H))
+        self.o_w = _param(_rand(gen, hidden, H * Dv, std=1.0 / math.sqrt(H * Dv), dtype=dtype))
+        self.register_buffer("inv_freq", mx.rotary_inv_freq(m.rot_dims, m.rot_base).to(dev),
+                             persistent=False)
+
+    def kv_shape(self):
+        # one key head of kv_rank + rot_dim channels; the values are its
+        # first kv_rank channels and take no storage of their own
+        return (1, self.R + self.rot, self.R, "prefix") if self.own else None
+
+    def state_shapes(self) -> Dict[str, tuple]:
+        return {}
+
+    def forward(self, h, sb: mx.SeqBatch, kv, state) -> torch.Tensor:
+        k_cache, v_view = kv
+        T = h.shape[0]
+        H, D, Dv, R, rot = self.H, self.D, self.Dv, self.R, self.rot
+        proj = ops.linear(h, self.proj_w)                     # [T, q | dkv | gate]
+        if self.own:
+            mx.latent_kv_prepare(proj[:, self.n_q : self.n_q + self.n_kv], self.dkv_norm_w,
+                                 self.inv_freq, R, rot, self.eps, k_cache, sb)
+        q = proj[:, : self.n_q]
+        q_un = q.view(T, H, D + rot)[..., :D].transpose(0, 1)  # [H, T, D]
+        q_lat = torch.bmm(q_un, self.uk_w)                    # [H, T, R]
+        qf = mx.latent_q_assemble(q, q_lat, self.inv_freq, H, D, rot, sb)
+        ctx = mx.attention_paged(qf, k_cache, v_view, sb, self.scale, sinks=self.sinks,
+                                 gate_logits=proj[:, self.n_q + self.n_kv :])
+        val = torch.bmm(ctx.view(T, H, R).transpose(0, 1), self.uv_w.transpose(1, 2))
+        return ops.linear(val.transpose(0, 1).reshape(T, H * Dv), self.o_w)
+
+    def load(self, get, put, p: str) -> None:
+        parts = [get(p + "q")] + ([get(p + "dkv")] if self.own else []) + [get(p + "g")]
+        put(self.proj_w, parts)
+        if self.own:
+            put(self.dkv_norm_w, [get(p + "dkv.norm")])
+        self.uk_w.data.copy_(get(p + "uk").reshape(self.H, self.D, self.R)
+                             .to(self.uk_w.device, self.uk_w.dtype))
+        self.uv_w.data.copy_(get(p + "uv").reshape(self.H, self.Dv, self.R)
+                             .to(self.uv_w.device, self.uv_w.dtype))
+        put(self.sinks, [get(p + "sink")])
+        put(self.o_w, [get(p + "o")])
+
+
+class LightningMixer(nn.Module):
+    """Linear attention with one fixed decay per head: q, k (heads x dim) and
+    v (heads x vdim) pass silu; per head S <- decay_h S + k v^T, o = S^T q
+    with S float32 per-sequence state. The concatenated heads are RMS-normed
+    as one vector (weight [heads * vdim]) and gated by sigmoid(W_g h).
+
+    Fused projection rows: q | k | v | gate."""
+
+    def __init__(self, hidden: int, m: MixerSpec, eps: float, dtype, gen):
+        super().__init__()
+        self.H, self.D, self.Dv = m.heads, m.dim, m.vdim
+        self.eps, self.dtype = eps, dtype
+        H, D, Dv = self.H, self.D, self.Dv
+        self.proj_w = _param(_rand(gen, 2 * H * D + 2 * H * Dv, hidden,
+                                   std=1.0 / math.sqrt(hidden), dtype=dtype))
+        self.norm_w = _param(1.0 + 0.1 * _rand(gen, H * Dv))
+        self.o_w = _param(_rand(gen, hidden, H * Dv, std=1.0 / math.sqrt(H * Dv), dtype=dtype))
+        self.register_buffer(
+            "decay", torch.tensor([float(d) for d in m.decay], dtype=torch.float64)
+            .to(torch.float32).to(gen.device), persistent=False)
+
+    def kv_shape(self):
+        return None
+
+    def state_shapes(self) -> Dict[str, tuple]:
+        return {"S": (self.H, self.Dv, self.D)}      # S transposed: [head, value, key]
+
+    def forward(self, h, sb: mx.SeqBatch, kv, state) -> torch.Tensor:
+        n, nv = self.H * self.D, self.H * self.Dv
+        proj = ops.linear(h, self.proj_w)
+        o = mx.decay_linear_attention(proj[:, :n], proj[:, n : 2 * n], proj[:, 2 * n : 2 * n + nv],
+                                      state["S"], sb, self.H, self.D, self.Dv,
+                                      head_decay=self.decay, act="silu")
+        y = mx.gated_rms_norm(o, self.norm_w, 1, proj[:, 2 * n + nv :], "sigmoid", self.eps,
+                              self.dtype)
+        return ops.linear(y, self.o_w)
+
+    def load(self, get, put, p: str) -> None:
+        put(self.proj_w, [get(p + "q"), get(p + "k"), get(p + "v"), get(p + "g")])
+        put(self.norm_w, [get(p + "norm")])
+        put(self.o_w, [get(p + "o")])
+
+
+class GatedLinearAttentionMixer(nn.Module):
+    """Linear attention with a learned decay per head and key channel:
+    q = W_q h * dim^-1/2, k = W_k h, v = W_v h; a = sigmoid(W_a2 W_a1 h +
+    b)^(1/tau) (float32); per head S <- diag(a) S + k v^T, o = S^T q with S
+    float32 per-sequence state. Each head's o is RMS-normed over vdim (weight
+    [vdim], the same for every head) and gated by silu(W_g h).
+
+    Fused projection rows: q | k | v | gate | a1."""
+
+    def __init__(self, hidden: int, m: MixerSpec, eps: float, dtype, gen):
+        super().__init__()
+        self.H, self.D, self.Dv = m.heads, m.dim, m.vdim
+        self.eps, self.dtype = eps, dtype
+        self.inv_tau = 1.0 / float(m.tau)
+        self.ra = m.decay_rank or max(4, hidden // 16)
+        H, D, Dv = self.H, self.D, self.Dv
+        self.proj_w = _param(_rand(gen, 2 * H * D + 2 * H * Dv + self.ra, hidden,
+                                   std=1.0 / math.sqrt(hidden), dtype=dtype))
+        self.a2_w = _param(_rand(gen, H * D, self.ra, std=1.0 / math.sqrt(self.ra), dtype=dtype))
+        self.a2_b = _param(_rand(gen, H * D) + 2.0)
+        self.norm_w = _param(1.0 + 0.1 * _rand(gen, Dv))
+        self.o_w = _param(_rand(gen, hidden, H * Dv, std=1.0 / math.sqrt(H * Dv), dtype=dtype))
+
+    def kv_shape(self):
+        return None
+
+    def state_shapes(self) -> Dict[str, tuple]:
+        return {"S": (self.H, self.Dv, self.D)}
+
+    def forward(self, h, sb: mx.SeqBatch, kv, state) -> torch.Tensor:
+        n, nv = self.H * self.D, self.H * self.Dv
+        proj = ops.linear(h, self.proj_w)
+        z = ops.linear(proj[:, 2 * n + 2 * nv :], self.a2_w)  # [T, H*D]
+        o = mx.decay_linear_attention(proj[:, :n], proj[:, n : 2 * n], proj[:, 2 * n : 2 * n + nv],
+                                      state["S"], sb, self.H, self.D, self.Dv, z=z,
+                                      z_bias=self.a2_b, inv_tau=self.inv_tau,
+                                      q_scale=self.D ** -0.5)
+        y = mx.gated_rms_norm(o, self.norm_w, self.H, proj[:, 2 * n + nv : 2 * n + 2 * nv],
+                              "silu", self.eps, self.dtype)
+        return ops.linear(y, self.o_w)
+
+    def load(self, get, put, p: str) -> None:
+        put(self.proj_w, [get(p + "q"), get(p + "k"), get(p + "v"), get(p + "g"), get(p + "a1")])
+        put(self.a2_w, [get(p + "a2")])
+        put(self.a2_b, [get(p + "a2.b")])
+        put(self.norm_w, [get(p + "norm")])
+        put(self.o_w, [get(p + "o")])
+
+
 MIXERS = {"attention": BiasedAttentionMixer, "channel_delta": ChannelDeltaMixer,
-          "rotary_window": RotaryWindowAttentionMixer}
+          "rotary_window": RotaryWindowAttentionMixer,
+          "latent_attention": LatentAttentionMixer, "lightning": LightningMixer,
+          "gla": GatedLinearAttentionMixer}
 
 
 class GatedMLP(nn.Module):
-    """down(act(gate x) * (up x)); gate|up fused; act "silu" | "gelu_tanh"."""
+    """down(act(gate x) * (up x)); gate|up fused; act "silu" | "gelu_tanh" |
+    ("clamp_swish", limit, alpha)."""
 
     def __init__(self, hidden: int, ff: int, dtype, gen, act: str = "silu"):
         super().__init__()
@@ -233,6 +418,7 @@ class GatedMLP(nn.Module):
         M, K = x.shape
         if (
             x.is_cuda and x.dtype == torch.bfloat16 and K % 8 == 0 and self.ff % 8 == 0
+            and isinstance(self.act, str)
             and (ops._gemv_m_ok(M) or ops._bf16_mfma_ok(M, K, gateup=True))
         ):
             act = ops.gateup_act(x, self.gate_up_w, self.ff, self.act)   # fused decode GEMV
@@ -348,7 +534,60 @@ class SandwichLayer(nn.Module):
             self.mlp.load(get, put, p + "mlp.")
 
 
-LAYER_STYLES = {"post_canon": HybridLayer, "sandwich": SandwichLayer}
+class PreNormLayer(nn.Module):
+    """x <- x + mixer(ln1(x));  x <- x + ff(ln2(x)) with weighted layer norms
+    (no bias; float32 weights and statistics). The add after a sublayer and
+    the norm before the next one (also the next layer's) are one launch:
+    forward takes the already-normed mixer input and returns the next
+    layer's. A routed feed-forward hands its routed sum, its shared expert's
+    output and that expert's gate logits to the same launch."""
+
+    def __init__(self, spec: HybridSpec, ls: HybridLayerSpec, dtype, gen):
+        super().__init__()
+        C = spec.hidden_size
+        self.dtype, self.eps = dtype, spec.norm_eps
+        self.norm1_w = _param(1.0 + 0.05 * _rand(gen, C))
+        self.mixer = MIXERS[ls.mixer.kind](C, ls.mixer, spec.norm_eps, dtype, gen)
+        self.mlp = None
+        if ls.mlp_kind == "dense":
+            self.mlp = GatedMLP(C, ls.mlp_ff, dtype, gen, act=ls.mlp_act)
+        elif ls.mlp_kind == "moe":
+            from opsagent_amd.engine.moe import RoutedExperts
+
+            self.mlp = RoutedExperts(C, ls.router, dtype, gen)
+        self.routed = ls.mlp_kind == "moe"
+        if self.mlp is not None:
+            self.norm2_w = _param(1.0 + 0.05 * _rand(gen, C))
+
+    def state_shapes(self) -> Dict[str, tuple]:
+        return dict(self.mixer.state_shapes())
+
+    def first_norm(self):
+        return self.norm1_w
+
+    def forward(self, x, h, sb: mx.SeqBatch, kv, state, next_norm):
+        """x: float32 residual [T, C] (updated in place); h = ln1(x).
+        next_norm: the following layer's first norm weight (None after the
+        last layer). Returns (x, next layer's h or None)."""
+        y = self.mixer(h, sb, kv, state)
+        if self.mlp is None:
+            return x, mx.add_layer_norm(x, next_norm, self.eps, self.dtype, y=y)
+        h2 = mx.add_layer_norm(x, self.norm2_w, self.eps, self.dtype, y=y)
+        if self.routed:
+            m, shared, gate = self.mlp.forward_parts(h2, decode=sb.max_chunk == 1)
+            return x, mx.add_layer_norm(x, next_norm, self.eps, self.dtype, y=m, y2=shared,
+                                        y2_gate=gate)
+        return x, mx.add_layer_norm(x, next_norm, self.eps, self.dtype, y=self.mlp(h2))
+
+    def load(self, get, put, p: str) -> None:
+        put(self.norm1_w, [get(p + "norm1")])
+        self.mixer.load(get, put, p + "mix.")
+        if self.mlp is not None:
+            put(self.norm2_w, [get(p + "norm2")])
+            self.mlp.load(get, put, p + "mlp.")
+
+
+LAYER_STYLES = {"post_canon": HybridLayer, "sandwich": SandwichLayer, "pre_norm": PreNormLayer}
 
 
 class HybridForCausalLM(nn.Module):
@@ -365,13 +604,19 @@ class HybridForCausalLM(nn.Module):
         C = spec.hidden_size
         self.embed = _param(_rand(gen, spec.vocab_size, C, dtype=dtype))
         self.sandwich = spec.layer_style == "sandwich"
+        self.pre_norm = spec.layer_style == "pre_norm"
         self.layers = nn.ModuleList(
             [LAYER_STYLES[spec.layer_style](spec, ls, dtype, gen) for ls in spec.layers]
         )
         if self.sandwich:
             self.final_norm = DyTNorm(C, gen)
+        elif self.pre_norm:
+            self.final_norm_w = _param(torch.ones(C, device=device))
         else:
             self.final_norm_w = _param(torch.ones(C, dtype=dtype, device=device))
+        # layer i reads the cache of layer kv_source[i] (its own unless its
+        # mixer names another layer)
+        self.kv_source = [getattr(layer.mixer, "kv_source", None) for layer in self.layers]
         self.lm_head = _param(_rand(gen, spec.vocab_size, C, std=1.0 / math.sqrt(C), dtype=dtype))
         self.vocab_local = spec.vocab_size
         self.to(device)
@@ -388,13 +633,18 @@ class HybridForCausalLM(nn.Module):
     def forward(self, fb: ForwardBatch, kv_caches, state=None) -> torch.Tensor:
         sb = fb.seq_batch
         assert sb is not None and state is not None, "hybrid models run flat multi-sequence steps"
-        x = mx.embed_rows(self.embed, fb.input_ids)
-        if self.sandwich:
+        x = mx.embed_rows(self.embed, fb.input_ids, self.spec.embed_scale)
+        if self.sandwich or self.pre_norm:
             n = len(self.layers)
-            h = mx.dyt_norm(x, self.layers[0].first_norm(), self.dtype)
+            if self.sandwich:
+                h = mx.dyt_norm(x, self.layers[0].first_norm(), self.dtype)
+            else:
+                h = mx.add_layer_norm(x, self.layers[0].first_norm(), self.spec.norm_eps,
+                                      self.dtype)
             for i, layer in enumerate(self.layers):
                 nxt = self.layers[i + 1].first_norm() if i + 1 < n else None
-                x, h = layer(x, h, sb, kv_caches[i], state[i], nxt)
+                src = self.kv_source[i]
+                x, h = layer(x, h, sb, kv_caches[i if src is None else src], state[i], nxt)
                 if self.trace_layers is not None:
                     self.trace_layers.append(x.clone())
             return x
@@ -409,6 +659,9 @@ class HybridForCausalLM(nn.Module):
         if the design caps them)."""
         if self.sandwich:
             normed = mx.dyt_norm(hidden.contiguous(), self.final_norm.params(), self.dtype)
+        elif self.pre_norm:
+            normed = mx.add_layer_norm(hidden.contiguous(), self.final_norm_w,
+                                       self.spec.norm_eps, self.dtype)
         else:
             _, normed = mx.group_rms_norm(hidden, self.final_norm_w, self.spec.norm_groups,
                                           self.spec.norm_eps, residual=None)
@@ -441,8 +694,11 @@ class HybridForCausalLM(nn.Module):
 
         put(self.embed, [get("embed")])
         put(self.lm_head, [get("head")])
-        if self.sandwich:
-            self.final_norm.load(get, put, "final.norm")
+        if self.sandwich or self.pre_norm:
+            if self.sandwich:
+                self.final_norm.load(get, put, "final.norm")
+            else:
+                put(self.final_norm_w, [get("final.norm")])
             for i, layer in enumerate(self.layers):
                 layer.load(get, put, f"l{i}.")
             return n

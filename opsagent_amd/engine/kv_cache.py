@@ -41,8 +41,11 @@ class PagedKVCache:
     ):
         """layer_shapes (optional) gives each layer's own (kv_heads, key dim,
         value dim), or None for a layer that keeps no keys and values (a
-        recurrent mixer); without it every layer is [kv_heads, head_dim] for
-        both. prefix_caching=False turns block publishing and reuse off: a
+        recurrent mixer, or a layer that reads another layer's cache); a
+        fourth element "prefix" says that the values ARE the first `value
+        dim` channels of the keys (one key head): the value tensor is then a
+        view of the key rows and takes no memory. Without layer_shapes every
+        layer is [kv_heads, head_dim] for both. prefix_caching=False turns block publishing and reuse off: a
         model that also carries recurrent state cannot restart from cached
         keys alone."""
         assert block_size & (block_size - 1) == 0, "block_size must be a power of 2"
@@ -57,9 +60,13 @@ class PagedKVCache:
             if shape is None:
                 self.layers.append((None, None))
                 continue
-            hk, kdim, vdim = shape
+            hk, kdim, vdim = shape[:3]
             k = torch.zeros(num_blocks, block_size, hk, kdim, dtype=dtype, device=device)
-            v = torch.zeros(num_blocks, block_size, hk, vdim, dtype=dtype, device=device)
+            if len(shape) > 3 and shape[3] == "prefix":
+                assert hk == 1 and vdim <= kdim
+                v = k[..., :vdim]
+            else:
+                v = torch.zeros(num_blocks, block_size, hk, vdim, dtype=dtype, device=device)
             self.layers.append((k, v))
         # allocator state
         self._free: collections.deque[int] = collections.deque(range(num_blocks))

@@ -12,6 +12,8 @@ token gather/scatter. The CDNA4 fp8-MFMA expert GEMM kernel (spec.moe_dtype
 
 from __future__ import annotations
 
+from typing import Optional
+
 import torch
 import torch.nn.functional as F
 from torch import nn
@@ -177,9 +179,13 @@ class MoEMLP(nn.Module):
 class RoutedExperts(nn.Module):
     """Mixture of gated feed-forwards with a score-and-choose router whose
     every constant is a RouterSpec field: sigmoid (or softmax) scores, a
-    learned correction that enters the CHOICE only, group-limited choice,
-    weights normalised over the chosen experts and scaled, an optional
-    always-on shared expert. Router logits, scores and weights are float32.
+    learned correction that enters the CHOICE only, group-limited choice
+    (groups rated by their two best scores or their best one), weights
+    normalised over the chosen experts (or not) and scaled, the experts'
+    gate activation with its constants, an optional always-on shared expert
+    with an optional per-token sigmoid gate whose projection is one more row
+    of the float32 router matrix. Router logits, scores and weights are
+    float32.
 
     Expert weights are stacked: w13 [E, 2I, C] (gate rows, then up rows) and
     w2 [E, C, I]. Few (token, expert) pairs run through two static-shaped
@@ -188,36 +194,60 @@ class RoutedExperts(nn.Module):
     """
 
     def __init__(self, hidden: int, r, dtype: torch.dtype, gen: torch.Generator,
-                 act: str = "silu"):
+                 act: Optional[str] = None):
         super().__init__()
         if get_tp_size() != 1:
             raise NotImplementedError("routed experts run at tensor-parallel size 1")
         from opsagent_amd.engine.hybrid import GatedMLP, _param, _rand
 
+        act = act or r.act
+        shared_act = act
+        if act == "clamp_swish":
+            act = ("clamp_swish", float(r.limit), float(r.alpha))
+            shared_act = ("clamp_swish", float(r.shared_limit or r.limit), float(r.alpha))
         self.r, self.act, self.hidden = r, act, hidden
         E, I = r.experts, r.ff
-        self.router_w = _param(_rand(gen, E, hidden, std=hidden ** -0.5))
+        self.shared_gate = bool(r.shared_gate and r.shared_ff)
+        # router rows, then (optionally) the shared expert's gate row
+        self.router_w = _param(_rand(gen, E + int(self.shared_gate), hidden, std=hidden ** -0.5))
         self.correction = _param(0.1 * _rand(gen, E)) if r.correction else None
         self.w13 = _param(_rand(gen, E, 2 * I, hidden, std=hidden ** -0.5, dtype=dtype))
         self.w2 = _param(_rand(gen, E, hidden, I, std=I ** -0.5, dtype=dtype))
-        self.shared = GatedMLP(hidden, r.shared_ff, dtype, gen, act=act) if r.shared_ff else None
+        self.shared = (GatedMLP(hidden, r.shared_ff, dtype, gen, act=shared_act)
+                       if r.shared_ff else None)
         # weight bytes one launch pair may stream through the pair kernels
         self.pair_budget = 64 << 20
         self.force_path = None     # "pairs" | "sorted" (tests)
 
-    def route(self, x: torch.Tensor):
+    def route(self, x: torch.Tensor, with_gate: bool = False):
         from opsagent_amd.ops import mixer_ops as mx
 
         logits = F.linear(x.float(), self.router_w)
-        return mx.route_topk(logits, self.correction, self.r.top, self.r.groups, self.r.keep,
-                             self.r.scale, self.r.score)
+        E = self.r.experts
+        idx, wts = mx.route_topk(logits[:, :E], self.correction, self.r.top, self.r.groups,
+                                 self.r.keep, self.r.scale, self.r.score, self.r.rating,
+                                 self.r.renorm)
+        if with_gate:
+            return idx, wts, (logits[:, E] if self.shared_gate else None)
+        return idx, wts
 
     def forward(self, x: torch.Tensor, decode: bool = False) -> torch.Tensor:
         """decode: the step holds one token per sequence; such batches stay on
         the static-shaped pair kernels up to 2048 pairs, so the step can be
         captured in a hipGraph."""
+        out, shared, gate = self.forward_parts(x, decode)
+        if shared is not None:
+            if gate is not None:
+                shared = (torch.sigmoid(gate).unsqueeze(1) * shared.float()).to(out.dtype)
+            out = out + shared
+        return out
+
+    def forward_parts(self, x: torch.Tensor, decode: bool = False):
+        """(routed sum, shared expert's output or None, float32 gate logits
+        [T] of the shared expert or None): a caller that adds them to a
+        residual can do so in one launch."""
         T, C = x.shape
-        idx, wts = self.route(x)
+        idx, wts, gate = self.route(x, with_gate=True)
         P, I = T * self.r.top, self.r.ff
         esz = 4 if x.dtype == torch.float32 else 2
         pairs = (P <= 64 or P * 3 * I * C * esz <= self.pair_budget
@@ -228,9 +258,7 @@ class RoutedExperts(nn.Module):
             out = self._pairs(x, idx, wts)
         else:
             out = self._sorted(x, idx, wts)
-        if self.shared is not None:
-            out = out + self.shared(x)
-        return out
+        return out, (self.shared(x) if self.shared is not None else None), gate
 
     def _pairs(self, x, idx, wts):
         from opsagent_amd.ops import mixer_ops as mx
@@ -278,7 +306,8 @@ class RoutedExperts(nn.Module):
 
     def load(self, get, put, p: str) -> None:
         E = self.r.experts
-        put(self.router_w, [get(p + "router")])
+        put(self.router_w, [get(p + "router")]
+            + ([get(p + "shared.sg")] if self.shared_gate else []))
         if self.correction is not None:
             put(self.correction, [get(p + "correction")])
         w13 = torch.stack([torch.cat([get(f"{p}e{k}.gate"), get(f"{p}e{k}.up")], 0)

@@ -369,22 +369,33 @@ extern "C" int oa_attn_rope_prepare(void* stream, const void* qkv, int64_t qs, c
 // ---------------------------------------------------------------------------
 // Gated activation over rows of [gate | up]: out = act(gate) * up.
 // act 0: silu g * sigmoid(g); act 1: gelu in its tanh approximation,
-// g/2 * (1 + tanh(k (g + 0.044715 g^3))), k = sqrt(2/pi). Evaluated in float32.
+// g/2 * (1 + tanh(k (g + 0.044715 g^3))), k = sqrt(2/pi); act 2: the clamped
+// form g' = min(g, limit), u' = clamp(u, -limit, limit),
+// out = g' sigmoid(alpha g') (u' + 1). Evaluated in float32.
 __device__ __forceinline__ float gate_act_f(float z, int act) {
     if (act == 1) return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
     return z / (1.0f + expf(-z));
+}
+__device__ __forceinline__ float gated_act_f(float g, float u, int act, float limit, float alpha) {
+    if (act == 2) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+        return g / (1.0f + expf(-alpha * g)) * (u + 1.0f);
+    }
+    return gate_act_f(g, act) * u;
 }
 
 template <typename TC>
 __global__ __launch_bounds__(256) void act_mul_rows_kernel(const TC* __restrict__ gu,
                                                            TC* __restrict__ out, int64_t M,
-                                                           int I, int act) {
+                                                           int I, int act, float limit,
+                                                           float alpha) {
     const int64_t total = M * I;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
          i += (int64_t)gridDim.x * blockDim.x) {
         const int64_t m = i / I;
         const int c = (int)(i % I);
-        stf(out, i, gate_act_f(ldf(gu, m * 2 * I + c), act) * ldf(gu, m * 2 * I + I + c));
+        stf(out, i, gated_act_f(ldf(gu, m * 2 * I + c), ldf(gu, m * 2 * I + I + c), act, limit, alpha));
     }
 }
 
@@ -392,7 +403,8 @@ __global__ __launch_bounds__(256) void act_mul_rows_kernel(const TC* __restrict_
 template <typename TC>
 __global__ __launch_bounds__(256) void act_mul_rows_vec_kernel(const TC* __restrict__ gu,
                                                                TC* __restrict__ out, int64_t M,
-                                                               int I, int act) {
+                                                               int I, int act, float limit,
+                                                               float alpha) {
     const int iv = I / 8;
     const int64_t total = M * iv;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
@@ -403,33 +415,33 @@ __global__ __launch_bounds__(256) void act_mul_rows_vec_kernel(const TC* __restr
         ld8(gu, m * 2 * I + c, g);
         ld8(gu, m * 2 * I + I + c, u);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) g[e] = gate_act_f(g[e], act) * u[e];
+        for (int e = 0; e < 8; ++e) g[e] = gated_act_f(g[e], u[e], act, limit, alpha);
         st8(out, m * I + c, g);
     }
 }
 
 extern "C" int oa_act_mul_rows(void* stream, const void* gu, void* out, int64_t M, int I, int dt,
-                               int act) {
+                               int act, float limit, float alpha) {
     if (M <= 0 || I <= 0) return 0;
-    if (act < 0 || act > 1) return -100;
+    if (act < 0 || act > 2) return -100;
     hipStream_t s = (hipStream_t)stream;
     const bool vec = I % 8 == 0 && (uintptr_t)gu % 32 == 0 && (uintptr_t)out % 32 == 0;
     if (vec) {
         const int grid = grid_for(M * (I / 8));
         if (dt == 1)
             hipLaunchKernelGGL((act_mul_rows_vec_kernel<float>), dim3(grid), dim3(256), 0, s,
-                               (const float*)gu, (float*)out, M, I, act);
+                               (const float*)gu, (float*)out, M, I, act, limit, alpha);
         else
             hipLaunchKernelGGL((act_mul_rows_vec_kernel<bf16s>), dim3(grid), dim3(256), 0, s,
-                               (const bf16s*)gu, (bf16s*)out, M, I, act);
+                               (const bf16s*)gu, (bf16s*)out, M, I, act, limit, alpha);
     } else {
         const int grid = grid_for(M * I);
         if (dt == 1)
             hipLaunchKernelGGL((act_mul_rows_kernel<float>), dim3(grid), dim3(256), 0, s,
-                               (const float*)gu, (float*)out, M, I, act);
+                               (const float*)gu, (float*)out, M, I, act, limit, alpha);
         else
             hipLaunchKernelGGL((act_mul_rows_kernel<bf16s>), dim3(grid), dim3(256), 0, s,
-                               (const bf16s*)gu, (bf16s*)out, M, I, act);
+                               (const bf16s*)gu, (bf16s*)out, M, I, act, limit, alpha);
     }
     HIP_CHECK_LAUNCH();
     return 0;
@@ -466,13 +478,13 @@ __device__ __forceinline__ ArgMax wave_argmax(ArgMax a) {
 __global__ __launch_bounds__(64) void route_topk_kernel(
     const float* __restrict__ logits, const float* __restrict__ correction,
     int* __restrict__ idx_out, float* __restrict__ w_out, int E, int top, int groups, int keep,
-    float scale, int score) {
+    float scale, int score, int64_t ls, int rating, int renorm) {
     extern __shared__ float lds[];
     float* S = lds;
     float* Cc = S + E;
     float* Gs = Cc + E;
     const int t = blockIdx.x, lane = threadIdx.x;
-    const float* z = logits + (int64_t)t * E;
+    const float* z = logits + (int64_t)t * ls;
     if (score == 1) {
         float mx = -INFINITY;
         for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
@@ -499,7 +511,7 @@ __global__ __launch_bounds__(64) void route_topk_kernel(
                     b2 = c;
                 }
             }
-            Gs[g] = per > 1 ? a + b2 : a;
+            Gs[g] = (per > 1 && rating == 0) ? a + b2 : a;
         }
         __syncthreads();
         // mark the keep best groups by lifting them to +inf, one per round
@@ -543,14 +555,14 @@ __global__ __launch_bounds__(64) void route_topk_kernel(
         __syncthreads();
     }
     if (lane == 0) {
-        const float inv = scale / (wsum + 1e-20f);
+        const float inv = renorm ? scale / (wsum + 1e-20f) : scale;
         for (int r = 0; r < top; ++r) w_out[(int64_t)t * top + r] *= inv;
     }
 }
 
-extern "C" int oa_route_topk(void* stream, const void* logits, const void* correction, void* idx,
-                             void* w, int T, int E, int top, int groups, int keep, float scale,
-                             int score) {
+extern "C" int oa_route_topk(void* stream, const void* logits, int64_t ls, const void* correction,
+                             void* idx, void* w, int T, int E, int top, int groups, int keep,
+                             float scale, int score, int rating, int renorm) {
     if (T <= 0) return 0;
     if (E < 1 || top < 1 || top > E || groups < 1 || E % groups != 0 || keep < 1 ||
         keep > groups || (int64_t)keep * (E / groups) < top)
@@ -559,7 +571,7 @@ extern "C" int oa_route_topk(void* stream, const void* logits, const void* corre
     if (lds > 60 * 1024) return -101;
     hipLaunchKernelGGL(route_topk_kernel, dim3(T), dim3(64), lds, (hipStream_t)stream,
                        (const float*)logits, (const float*)correction, (int*)idx, (float*)w, E, top,
-                       groups, keep, scale, score);
+                       groups, keep, scale, score, ls, rating, renorm);
     HIP_CHECK_LAUNCH();
     return 0;
 }
@@ -602,7 +614,8 @@ __device__ __forceinline__ void dot2_rows(const TC* __restrict__ wa, const TC* _
 template <typename TC>
 __global__ __launch_bounds__(256) void moe_pairs_gateup_kernel(
     const TC* __restrict__ x, const TC* __restrict__ w13, const int* __restrict__ idx,
-    TC* __restrict__ mid, int top, int E, int I, int K, int act, int vec) {
+    TC* __restrict__ mid, int top, int E, int I, int K, int act, int vec, float limit,
+    float alpha) {
     const int p = blockIdx.x, t = p / top;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int e = min(max(idx[p], 0), E - 1);
@@ -611,7 +624,7 @@ __global__ __launch_bounds__(256) void moe_pairs_gateup_kernel(
     for (int r = blockIdx.y * 4 + wave; r < I; r += gridDim.y * 4) {
         float g, u;
         dot2_rows(we + (int64_t)r * K, we + (int64_t)(I + r) * K, xr, K, lane, vec != 0, g, u);
-        if (lane == 0) stf(mid, (int64_t)p * I + r, gate_act_f(g, act) * u);
+        if (lane == 0) stf(mid, (int64_t)p * I + r, gated_act_f(g, u, act, limit, alpha));
     }
 }
 
@@ -648,18 +661,18 @@ __global__ __launch_bounds__(256) void moe_pairs_down_kernel(
 
 extern "C" int oa_moe_pairs_gateup(void* stream, const void* x, const void* w13, const void* idx,
                                    void* mid, int T, int top, int E, int I, int K, int dt,
-                                   int act) {
+                                   int act, float limit, float alpha) {
     if (T <= 0) return 0;
-    if (top < 1 || E < 1 || I < 1 || K < 1 || act < 0 || act > 1) return -100;
+    if (top < 1 || E < 1 || I < 1 || K < 1 || act < 0 || act > 2) return -100;
     const int vec = (K % 8 == 0 && (uintptr_t)x % 32 == 0 && (uintptr_t)w13 % 32 == 0) ? 1 : 0;
     dim3 grid(T * top, std::min(CEIL_DIV(I, 4), 64));
     hipStream_t s = (hipStream_t)stream;
     if (dt == 1)
         hipLaunchKernelGGL((moe_pairs_gateup_kernel<float>), grid, dim3(256), 0, s, (const float*)x,
-                           (const float*)w13, (const int*)idx, (float*)mid, top, E, I, K, act, vec);
+                           (const float*)w13, (const int*)idx, (float*)mid, top, E, I, K, act, vec, limit, alpha);
     else
         hipLaunchKernelGGL((moe_pairs_gateup_kernel<bf16s>), grid, dim3(256), 0, s, (const bf16s*)x,
-                           (const bf16s*)w13, (const int*)idx, (bf16s*)mid, top, E, I, K, act, vec);
+                           (const bf16s*)w13, (const int*)idx, (bf16s*)mid, top, E, I, K, act, vec, limit, alpha);
     HIP_CHECK_LAUNCH();
     return 0;
 }

@@ -429,7 +429,8 @@ __global__ __launch_bounds__(256) void attn_bias_paged_kernel(
     const int* __restrict__ cu, const int* __restrict__ past,
     const int* __restrict__ block_table, int max_blocks, int block_size,
     const float* __restrict__ slopes, const float* __restrict__ sinks, int B, int H, int G,
-    int D, int Dv, int TQ, int KT, int kstride, float scale, int nsplit, int RB, int window) {
+    int D, int Dv, int TQ, int KT, int kstride, float scale, int nsplit, int RB, int window,
+    int64_t vrow) {
     extern __shared__ float lds[];
     // a block takes up to RB of the H/G query heads of one kv head
     const int hgroups = (H / G + RB - 1) / RB;
@@ -490,7 +491,7 @@ __global__ __launch_bounds__(256) void attn_bias_paged_kernel(
             const int j = i / Dv, d = i % Dv;
             const int key = k0 + j;
             const int64_t slot = (int64_t)bt[key / block_size] * block_size + key % block_size;
-            Vs[j * Dv + d] = v_cache[(slot * G + g) * Dv + d];
+            Vs[j * Dv + d] = v_cache[slot * vrow + g * Dv + d];
         }
         __syncthreads();
 #pragma unroll
@@ -596,7 +597,7 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
     const int* __restrict__ cu, const int* __restrict__ past,
     const int* __restrict__ block_table, int max_blocks, int block_size,
     const float* __restrict__ slopes, const float* __restrict__ sinks, int B, int H, int G,
-    int D, int Dv, int HB, float scale, int nsplit, int window) {
+    int D, int Dv, int HB, float scale, int nsplit, int window, int64_t vrow) {
     // NT: 16-token sub-tiles per wave. Every K and V fragment read from LDS
     // feeds NT MFMAs, and a staged tile serves NT times the query rows.
     extern __shared__ float lds[];
@@ -697,7 +698,7 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
         const int64_t sk_ = okk ? ((int64_t)bt[keyk >> bsh] << bsh) + (keyk & bmask) : 0;
         const int64_t sv_ = okv ? ((int64_t)bt[keyv >> bsh] << bsh) + (keyv & bmask) : 0;
         const bf16s* kp = k_cache + (sk_ * G + g) * D;
-        const bf16s* vp = v_cache + (sv_ * G + g) * Dv;
+        const bf16s* vp = v_cache + sv_ * vrow + g * Dv;
 #pragma unroll
         for (int u = 0; u < KC; ++u) {
             const int c = kc0 + 4 * u;
@@ -1195,12 +1196,12 @@ template <typename TC>
 __global__ __launch_bounds__(256) void embed_rows_kernel(const TC* __restrict__ table,
                                                          const int64_t* __restrict__ ids,
                                                          float* __restrict__ out, int T,
-                                                         int C) {
+                                                         int C, float scale) {
     const int64_t total = (int64_t)T * C;
     for (int64_t idx = blockIdx.x * (int64_t)blockDim.x + threadIdx.x; idx < total;
          idx += (int64_t)gridDim.x * blockDim.x) {
         const int t = (int)(idx / C), c = (int)(idx % C);
-        out[idx] = ldf(table, ids[t] * (int64_t)C + c);
+        out[idx] = ldf(table, ids[t] * (int64_t)C + c) * scale;
     }
 }
 
@@ -1398,7 +1399,7 @@ static void launch_attn_mfma(hipStream_t s, dim3 grid, int lds_bytes, const void
                              void* part_o, void* part_ml, const void* cu, const void* past,
                              const void* block_table, int max_blocks, int block_size,
                              const void* slopes, const void* sinks, int B, int H, int G, int D,
-                             int Dv, int HB, float scale, int nsplit, int window) {
+                             int Dv, int HB, float scale, int nsplit, int window, int64_t vrow) {
     if (lds_bytes > 48 * 1024)
         (void)hipFuncSetAttribute((const void*)attn_bias_mfma_kernel<MAXD, MAXDV, QK32, NT>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
@@ -1407,7 +1408,7 @@ static void launch_attn_mfma(hipStream_t s, dim3 grid, int lds_bytes, const void
                        (const bf16s*)v_cache, (bf16s*)out, (float*)part_o, (float*)part_ml,
                        (const int*)cu, (const int*)past, (const int*)block_table, max_blocks,
                        block_size, (const float*)slopes, (const float*)sinks, B, H, G, D, Dv, HB,
-                       scale, nsplit, window);
+                       scale, nsplit, window, vrow);
 }
 
 // ntiles = sum_b ceil(n_b / TQ) (host-computed). part_* may be null when nsplit == 1.
@@ -1417,20 +1418,25 @@ extern "C" int oa_attn_bias_paged(void* stream, const void* q, const void* gate,
                                   const void* block_table, int max_blocks, int block_size,
                                   const void* slopes, const void* sinks, int T, int B, int ntiles,
                                   int H, int G, int D, int Dv, float scale, int nsplit, int dt,
-                                  int max_chunk, int window) {
+                                  int max_chunk, int window, int64_t vrow) {
+    // vrow: elements between the value rows of consecutive cache slots
+    // (G * Dv for a cache of its own; more when the values are the leading
+    // channels of wider rows)
     if (T <= 0 || ntiles <= 0) return 0;
     if (window < 0) return -105;
+    if (vrow < (int64_t)G * Dv) return -106;
     int TQ, KT, ks, lds_bytes;
     int rc = oa_attn_bias_geometry(H, G, D, Dv, dt, max_chunk, &TQ, &KT, &ks, &lds_bytes);
     if (rc) return rc;
     if (nsplit < 1 || (nsplit > 1 && (!part_o || !part_ml))) return -104;
     hipStream_t s = (hipStream_t)stream;
     if (attn_path(H, G, D, Dv, dt)) {
+        if (vrow % 8 != 0) return -107;   // 16-byte value loads
         const int R = H / G, HB = attn_hb(R);
         dim3 grid(ntiles, G * (R / HB), nsplit);
 #define MF_ARGS                                                                                   \
     s, grid, lds_bytes, q, gate, gs, k_cache, v_cache, out, part_o, part_ml, cu, past, block_table, \
-        max_blocks, block_size, slopes, sinks, B, H, G, D, Dv, HB, scale, nsplit, window
+        max_blocks, block_size, slopes, sinks, B, H, G, D, Dv, HB, scale, nsplit, window, vrow
 #define MF(A, Bv)                                                               \
     do {                                                                        \
         if (D % 32 == 0) launch_attn_mfma<A, Bv, true, 1>(MF_ARGS);             \
@@ -1456,7 +1462,7 @@ extern "C" int oa_attn_bias_paged(void* stream, const void* q, const void* gate,
     (const TC*)q, (const TC*)gate, gs, (const TC*)k_cache, (const TC*)v_cache, (TC*)out,  \
         (float*)part_o, (float*)part_ml, (const int*)cu, (const int*)past,                \
         (const int*)block_table, max_blocks, block_size, (const float*)slopes,            \
-        (const float*)sinks, B, H, G, D, Dv, TQ, KT, ks, scale, nsplit, rb, window
+        (const float*)sinks, B, H, G, D, Dv, TQ, KT, ks, scale, nsplit, rb, window, vrow
         if (dt == 1)
             hipLaunchKernelGGL((attn_bias_paged_kernel<float>), grid, blk, lds_bytes, s, AT_ARGS(float));
         else
@@ -1571,15 +1577,15 @@ extern "C" int oa_silu_mul_rows(void* stream, const void* gu, void* out, int64_t
 }
 
 extern "C" int oa_embed_rows(void* stream, const void* table, const void* ids, void* out, int T,
-                             int C, int dt) {
+                             int C, int dt, float scale) {
     if (T <= 0) return 0;
     hipStream_t s = (hipStream_t)stream;
     if (dt == 1)
         hipLaunchKernelGGL((embed_rows_kernel<float>), dim3(grid_for((int64_t)T * C)), dim3(256), 0, s,
-                           (const float*)table, (const int64_t*)ids, (float*)out, T, C);
+                           (const float*)table, (const int64_t*)ids, (float*)out, T, C, scale);
     else
         hipLaunchKernelGGL((embed_rows_kernel<bf16s>), dim3(grid_for((int64_t)T * C)), dim3(256), 0, s,
-                           (const bf16s*)table, (const int64_t*)ids, (float*)out, T, C);
+                           (const bf16s*)table, (const int64_t*)ids, (float*)out, T, C, scale);
     HIP_CHECK_LAUNCH();
     return 0;
 }

@@ -125,19 +125,25 @@ def _declare_mixers(lib: ctypes.CDLL) -> None:
         "oa_attn_prepare": [p, p, i64, p, p, p, p, p, p, p, p, i, i, i, i, i, i, f, i],
         "oa_attn_bias_geometry": [i, i, i, i, i, i, ip, ip, ip, ip],
         "oa_attn_bias_paged": [p, p, p, i64, p, p, p, p, p, p, p, p, i, i, p, p,
-                               i, i, i, i, i, i, i, f, i, i, i, i],
+                               i, i, i, i, i, i, i, f, i, i, i, i, i64],
         "oa_dyt_norm": [p, p, i64, i, p, p, p, p, p, p, p, p, i, i, i],
         "oa_attn_rope_prepare": [p, p, i64, p, p, p, i, p, p, p, p, p, p, p, i, i,
                                  i, i, i, i, f, i],
-        "oa_act_mul_rows": [p, p, p, i64, i, i, i],
-        "oa_route_topk": [p, p, p, p, p, i, i, i, i, i, f, i],
-        "oa_moe_pairs_gateup": [p, p, p, p, p, i, i, i, i, i, i, i],
+        "oa_act_mul_rows": [p, p, p, i64, i, i, i, f, f],
+        "oa_route_topk": [p, p, i64, p, p, p, i, i, i, i, i, f, i, i, i],
+        "oa_moe_pairs_gateup": [p, p, p, p, p, i, i, i, i, i, i, i, f, f],
+        "oa_add_layer_norm": [p, p, p, i64, i, p, i64, i, p, i64, p, p, i, i, i, f],
+        "oa_latent_kv_prepare": [p, p, i64, p, p, i, p, p, p, p, p, i, i, i, i, f, i],
+        "oa_latent_q_assemble": [p, p, i64, p, p, i, p, p, p, p, i, i, i, i, i, i, i],
+        "oa_decay_scan": [p, p, i64, p, i64, p, i64, p, i64, p, f, p, p, p, p, p, p,
+                          i, i, i, i, i, i, f, i, i],
+        "oa_gated_rms_norm": [p, p, p, i, p, i64, i, i, p, i, i, i, i, f],
         "oa_moe_pairs_down": [p, p, p, p, p, p, i, i, i, i, i, i],
         "oa_delta_rule_fused": [p, p, i64, p, i64, p, i64, p, i64, p, i64, p, p, p, p, i64,
                                 p, p, p, p, p, p, i, i, i, i, i, i, f, i, i],
         "oa_softcap": [p, p, p, i64, f, i],
         "oa_silu_mul_rows": [p, p, p, i64, i, i],
-        "oa_embed_rows": [p, p, p, p, i, i, i],
+        "oa_embed_rows": [p, p, p, p, i, i, i, f],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)

@@ -96,16 +96,16 @@ def _rows(t: torch.Tensor) -> int:
     return t.stride(0)
 
 
-def embed_rows(table: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
-    """table[ids] as a float32 residual stream [T, C]."""
+def embed_rows(table: torch.Tensor, ids: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """table[ids] * scale as a float32 residual stream [T, C]."""
     if not table.is_cuda:
-        return table[ids].float()
+        return table[ids].float() * scale if scale != 1.0 else table[ids].float()
     lib, hip = _lib()
     T, C = ids.shape[0], table.shape[1]
     out = torch.empty(T, C, dtype=torch.float32, device=table.device)
     assert ids.dtype == torch.int64 and table.is_contiguous()
     hip.check(lib.oa_embed_rows(hip.current_stream_ptr(), table.data_ptr(), ids.data_ptr(),
-                                out.data_ptr(), T, C, _dt(table)), "oa_embed_rows")
+                                out.data_ptr(), T, C, _dt(table), float(scale)), "oa_embed_rows")
     return out
 
 
@@ -213,6 +213,10 @@ def attention_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     T, H, D = q.shape
     nb, bs, G, Dv = v_cache.shape
     window = int(window) if window else 0
+    # v_cache may be a view of the leading channels of wider rows (values
+    # that are a prefix of the cached keys): its token stride is passed on
+    assert v_cache.stride(3) == 1 and (G == 1 or v_cache.stride(2) == Dv)
+    assert v_cache.stride(0) == bs * v_cache.stride(1)
     if not q.is_cuda:
         return torch_ref.attention_paged(q, k_cache, v_cache, sb.cu, sb.past, sb.block_table,
                                          scale, slopes, gate_logits, window or None, sinks)
@@ -248,7 +252,7 @@ def attention_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         sb.block_table.shape[1], bs, slopes.data_ptr() if slopes is not None else None,
         sinks.data_ptr() if sinks is not None else None,
         T, sb.num_seqs, ntiles, H, G, D, Dv,
-        float(scale), nsplit, dt, sb.max_chunk, window)
+        float(scale), nsplit, dt, sb.max_chunk, window, v_cache.stride(1))
     hip.check(rc, "oa_attn_bias_paged")
     return out
 
@@ -345,12 +349,22 @@ def attn_rope_prepare(qkv: torch.Tensor, q_norm_w: torch.Tensor, k_norm_w: torch
     return q
 
 
-ACTS = {"silu": 0, "gelu_tanh": 1}
+ACTS = {"silu": 0, "gelu_tanh": 1, "clamp_swish": 2}
 
 
-def act_mul_rows(gu: torch.Tensor, inter: int, act: str = "silu") -> torch.Tensor:
+def act_args(act) -> Tuple[int, float, float]:
+    """(code, limit, alpha) of a gate activation given as a name or as
+    ("clamp_swish", limit, alpha)."""
+    if isinstance(act, tuple):
+        return ACTS[act[0]], float(act[1]), float(act[2])
+    return ACTS[act], 0.0, 0.0
+
+
+def act_mul_rows(gu: torch.Tensor, inter: int, act="silu") -> torch.Tensor:
     """act(gu[:, :I]) * gu[:, I:] for a contiguous [M, 2I] buffer; act is
-    "silu" or "gelu_tanh" (the tanh form of gelu), evaluated in float32."""
+    "silu", "gelu_tanh" (the tanh form of gelu) or ("clamp_swish", limit,
+    alpha): g = min(gate, limit), u = clamp(up, -limit, limit),
+    g sigmoid(alpha g) (u + 1); evaluated in float32."""
     if not gu.is_cuda:
         g, u = gu.split([inter, inter], dim=-1)
         return torch_ref.act_mul(g, u, act)
@@ -358,43 +372,47 @@ def act_mul_rows(gu: torch.Tensor, inter: int, act: str = "silu") -> torch.Tenso
     assert gu.is_contiguous() and gu.shape[-1] == 2 * inter
     M = gu.numel() // (2 * inter)
     out = torch.empty(*gu.shape[:-1], inter, dtype=gu.dtype, device=gu.device)
+    code, limit, alpha = act_args(act)
     hip.check(lib.oa_act_mul_rows(hip.current_stream_ptr(), gu.data_ptr(), out.data_ptr(),
-                                  M, inter, _dt(gu), ACTS[act]), "oa_act_mul_rows")
+                                  M, inter, _dt(gu), code, limit, alpha), "oa_act_mul_rows")
     return out
 
 
 def route_topk(logits: torch.Tensor, correction: Optional[torch.Tensor], top: int,
                groups: int = 1, keep: int = 1, scale: float = 1.0,
-               score: str = "sigmoid") -> Tuple[torch.Tensor, torch.Tensor]:
+               score: str = "sigmoid", rating: str = "top2",
+               renorm: bool = True) -> Tuple[torch.Tensor, torch.Tensor]:
     """Expert choice from float32 router logits [T, E]: returns (experts
     int32 [T, top], weights float32 [T, top]). score "sigmoid" | "softmax";
     c = score + correction (float32 [E], optional) ranks the experts; with
     groups > 1 the experts are cut into `groups` runs of E/groups neighbours,
-    each run is rated max1(c) + max2(c), and only the `keep` top-rated runs
-    may be picked from. Weights: w_j = scale * s_j / (sum_k s_k + 1e-20) over
-    the picked experts' uncorrected scores s."""
+    each run is rated max1(c) + max2(c) (rating "top2") or max(c) ("max"),
+    and only the `keep` top-rated runs may be picked from. Weights:
+    w_j = scale * s_j / (sum_k s_k + 1e-20) over the picked experts'
+    uncorrected scores s; renorm=False leaves out the division. logits may
+    be the leading columns of wider rows."""
     T, E = logits.shape
     assert logits.dtype == torch.float32 and E % max(groups, 1) == 0 and top <= E
     if groups > 1:
         assert keep * (E // groups) >= top, "too few eligible experts"
     if not logits.is_cuda:
-        return torch_ref.route_topk(logits, correction, top, groups, keep, scale, score)
+        return torch_ref.route_topk(logits, correction, top, groups, keep, scale, score,
+                                    rating, renorm)
     lib, hip = _lib()
-    logits = logits.contiguous()
     idx = torch.empty(T, top, dtype=torch.int32, device=logits.device)
     w = torch.empty(T, top, dtype=torch.float32, device=logits.device)
     assert correction is None or (correction.dtype == torch.float32 and correction.is_contiguous())
     rc = lib.oa_route_topk(
-        hip.current_stream_ptr(), logits.data_ptr(),
+        hip.current_stream_ptr(), logits.data_ptr(), _rows(logits),
         correction.data_ptr() if correction is not None else None, idx.data_ptr(),
         w.data_ptr(), T, E, top, max(groups, 1), keep, float(scale),
-        0 if score == "sigmoid" else 1)
+        0 if score == "sigmoid" else 1, 1 if rating == "max" else 0, int(bool(renorm)))
     hip.check(rc, "oa_route_topk")
     return idx, w
 
 
 def moe_pairs_mlp(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, idx: torch.Tensor,
-                  wts: torch.Tensor, act: str = "silu") -> torch.Tensor:
+                  wts: torch.Tensor, act="silu") -> torch.Tensor:
     """Routed experts for few tokens, two launches, no host sync and no
     atomics: out[t] = sum_j wts[t,j] * W2[e_tj] (act(Wg[e_tj] x_t) * (Wu[e_tj] x_t)).
     x [T, K]; w13 [E, 2I, K] (gate rows, then up rows); w2 [E, C, I]; idx
@@ -412,9 +430,10 @@ def moe_pairs_mlp(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, idx: tor
     assert w13.dtype == x.dtype and w2.dtype == x.dtype and w2.shape == (E, C, I)
     mid = torch.empty(T * top, I, dtype=x.dtype, device=x.device)
     out = torch.empty(T, C, dtype=x.dtype, device=x.device)
+    code, limit, alpha = act_args(act)
     hip.check(lib.oa_moe_pairs_gateup(
         hip.current_stream_ptr(), x.data_ptr(), w13.data_ptr(), idx.data_ptr(), mid.data_ptr(),
-        T, top, E, I, K, _dt(x), ACTS[act]), "oa_moe_pairs_gateup")
+        T, top, E, I, K, _dt(x), code, limit, alpha), "oa_moe_pairs_gateup")
     hip.check(lib.oa_moe_pairs_down(
         hip.current_stream_ptr(), mid.data_ptr(), w2.data_ptr(), idx.data_ptr(), wts.data_ptr(),
         out.data_ptr(), T, top, E, C, I, _dt(x)), "oa_moe_pairs_down")
@@ -471,6 +490,164 @@ def channel_delta_rule(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
         sb.past_t.data_ptr(), sb.slots_t.data_ptr(), T, sb.num_seqs, H, G, D, Dv, eps, _dt(q),
         csplit)
     hip.check(rc, "oa_delta_rule_fused")
+    return out
+
+
+def add_layer_norm(residual: torch.Tensor, w: Optional[torch.Tensor], eps: float, out_dtype,
+                   y: Optional[torch.Tensor] = None, y2: Optional[torch.Tensor] = None,
+                   y2_gate: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """One launch for the add after a sublayer and the layer norm before the
+    next: residual (float32 [T, C], in place) += y + sigmoid(y2_gate) * y2
+    (each optional; y2_gate float32 [T], may be a column of a wider buffer,
+    scales y2's rows; without it y2 is added as it is). With w (float32 [C]):
+    returns (x - mean) / sqrt(mean((x - mean)^2) + eps) * w of the new
+    residual in out_dtype; statistics in float32, two passes."""
+    T, C = residual.shape
+    assert residual.dtype == torch.float32 and residual.is_contiguous()
+    assert y2_gate is None or (y2 is not None and y2_gate.dtype == torch.float32
+                               and y2_gate.dim() == 1)
+    if not residual.is_cuda:
+        return torch_ref.add_layer_norm(residual, y, w, eps, out_dtype, y2, y2_gate)
+    lib, hip = _lib()
+    assert w is None or (w.dtype == torch.float32 and w.is_contiguous() and w.numel() == C)
+    out = torch.empty(T, C, dtype=out_dtype, device=residual.device) if w is not None else None
+    rc = lib.oa_add_layer_norm(
+        hip.current_stream_ptr(), residual.data_ptr(),
+        y.data_ptr() if y is not None else None, _rows(y) if y is not None else 0,
+        _dt(y) if y is not None else 1,
+        y2.data_ptr() if y2 is not None else None, _rows(y2) if y2 is not None else 0,
+        _dt(y2) if y2 is not None else 1,
+        y2_gate.data_ptr() if y2_gate is not None else None,
+        y2_gate.stride(0) if y2_gate is not None else 0,
+        w.data_ptr() if w is not None else None,
+        out.data_ptr() if out is not None else None, _dt(out) if out is not None else 1,
+        T, C, float(eps))
+    hip.check(rc, "oa_add_layer_norm")
+    return out
+
+
+def _positions(sb: SeqBatch) -> torch.Tensor:
+    return torch.tensor([sb.past[b] + i for b in range(sb.num_seqs)
+                         for i in range(sb.cu[b + 1] - sb.cu[b])], dtype=torch.float32)
+
+
+def latent_kv_prepare(dkv: torch.Tensor, norm_w: torch.Tensor, inv_freq: torch.Tensor,
+                      rank: int, rot: int, eps: float, k_cache: torch.Tensor,
+                      sb: SeqBatch) -> None:
+    """What latent attention caches per token, from dkv [T, rank + rot] (may
+    be a column slice): the first `rank` columns RMS-normed with the float32
+    weight norm_w (the latent), the last `rot` with channel pairs (2i, 2i+1),
+    i < len(inv_freq), rotated by position * inv_freq[i] (one key part for
+    all heads). Both go to the token's row of k_cache [blocks, page, 1,
+    rank + rot]; everything between load and store is float32."""
+    T = dkv.shape[0]
+    assert dkv.shape[1] == rank + rot and 2 * inv_freq.numel() <= rot
+    assert k_cache.shape[2:] == (1, rank + rot) and k_cache.is_contiguous()
+    if not dkv.is_cuda:
+        torch_ref.latent_kv_prepare(dkv, norm_w, inv_freq, rank, rot, eps, k_cache,
+                                    _positions(sb), sb.slot_mapping)
+        return
+    lib, hip = _lib()
+    assert k_cache.dtype == dkv.dtype
+    for t in (norm_w, inv_freq):
+        assert t.dtype == torch.float32 and t.is_contiguous()
+    rc = lib.oa_latent_kv_prepare(
+        hip.current_stream_ptr(), dkv.data_ptr(), _rows(dkv), norm_w.data_ptr(),
+        inv_freq.data_ptr(), inv_freq.numel(), k_cache.data_ptr(), sb.slot_mapping.data_ptr(),
+        sb.seq_of_t.data_ptr(), sb.cu_t.data_ptr(), sb.past_t.data_ptr(), sb.num_seqs, T,
+        rank, rot, float(eps), _dt(dkv))
+    hip.check(rc, "oa_latent_kv_prepare")
+
+
+def latent_q_assemble(q: torch.Tensor, q_lat: torch.Tensor, inv_freq: torch.Tensor,
+                      H: int, D: int, rot: int, sb: SeqBatch) -> torch.Tensor:
+    """Queries against the cached latent rows: q [T, H*(D+rot)] (per head D
+    unrotated, then rot rotated channels; may be a column slice) and q_lat
+    [H, T, rank], the unrotated parts already taken through the key
+    up-projection. Returns [T, H, rank + rot]: q_lat beside the part rotated
+    by position (float32 angles)."""
+    T = q.shape[0]
+    rank = q_lat.shape[2]
+    assert q_lat.shape[:2] == (H, T) and q_lat.is_contiguous() and q_lat.dtype == q.dtype
+    if not q.is_cuda:
+        return torch_ref.latent_q_assemble(q, q_lat, inv_freq, H, D, rot, _positions(sb))
+    lib, hip = _lib()
+    out = torch.empty(T, H, rank + rot, dtype=q.dtype, device=q.device)
+    rc = lib.oa_latent_q_assemble(
+        hip.current_stream_ptr(), q.data_ptr(), _rows(q), q_lat.data_ptr(),
+        inv_freq.data_ptr(), inv_freq.numel(), out.data_ptr(), sb.seq_of_t.data_ptr(),
+        sb.cu_t.data_ptr(), sb.past_t.data_ptr(), sb.num_seqs, T, H, D, rot, rank, _dt(q))
+    hip.check(rc, "oa_latent_q_assemble")
+    return out
+
+
+def decay_linear_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                           state: torch.Tensor, sb: SeqBatch, H: int, D: int, Dv: int,
+                           head_decay: Optional[torch.Tensor] = None,
+                           z: Optional[torch.Tensor] = None,
+                           z_bias: Optional[torch.Tensor] = None, inv_tau: float = 1.0,
+                           act: str = "none", q_scale: float = 1.0) -> torch.Tensor:
+    """Linear attention with decay: per head S_t = diag(a_t) S_{t-1} + k_t v_t^T,
+    o_t = S_t^T q_t. a_t is head_decay[h] (float32 [H]) for every key channel,
+    or, with z [T, H*D], sigmoid(z_t + z_bias)^(inv_tau) per key channel
+    (z_bias float32 [H*D]; computed as exp(inv_tau * log sigmoid) in
+    float32). act "silu" is applied to q, k, v first; q is then scaled by
+    q_scale. q, k [T, H*D], v [T, H*Dv] may be column slices. state [slots,
+    H, Dv, D] float32 (S transposed) is continued and updated; a sequence at
+    position 0 starts from zero whatever its slot holds. Returns the
+    read-out [T, H*Dv] float32."""
+    T = q.shape[0]
+    assert (head_decay is None) != (z is None)
+    assert state.dtype == torch.float32 and state.is_contiguous()
+    assert state.shape[1:] == (H, Dv, D)
+    if not q.is_cuda:
+        return torch_ref.decay_linear_attention(q, k, v, z, z_bias, inv_tau, head_decay, state,
+                                                sb.cu, sb.past, sb.slots, H, D, Dv, act, q_scale)
+    lib, hip = _lib()
+    for t in (head_decay, z_bias):
+        assert t is None or (t.dtype == torch.float32 and t.is_contiguous())
+    assert z is None or (z_bias is not None and z_bias.numel() == H * D)
+    assert head_decay is None or head_decay.numel() == H
+    out = torch.empty(T, H * Dv, dtype=torch.float32, device=q.device)
+    # one block per (sequence, head) holds all value columns; long portions
+    # of few sequences split the columns over blocks to fill the chip
+    csplit, pairs = 1, sb.num_seqs * H
+    if sb.max_chunk >= 64 and pairs < 192:
+        for c in (8, 4, 2):
+            if Dv % (4 * c) == 0 and Dv // c >= 16 and pairs * c <= 512:
+                csplit = c
+                break
+    rc = lib.oa_decay_scan(
+        hip.current_stream_ptr(), q.data_ptr(), _rows(q), k.data_ptr(), _rows(k),
+        v.data_ptr(), _rows(v), z.data_ptr() if z is not None else None,
+        _rows(z) if z is not None else 0,
+        z_bias.data_ptr() if z_bias is not None else None, float(inv_tau),
+        head_decay.data_ptr() if head_decay is not None else None, state.data_ptr(),
+        out.data_ptr(), sb.cu_t.data_ptr(), sb.past_t.data_ptr(), sb.slots_t.data_ptr(),
+        T, sb.num_seqs, H, D, Dv, 1 if act == "silu" else 0, float(q_scale), _dt(q), csplit)
+    hip.check(rc, "oa_decay_scan")
+    return out
+
+
+def gated_rms_norm(o: torch.Tensor, w: torch.Tensor, groups: int, gate_logits: torch.Tensor,
+                   gate_act: str, eps: float, out_dtype) -> torch.Tensor:
+    """o float32 [T, N]: RMS norm over each of `groups` equal parts, times the
+    float32 weight w ([N/groups], shared by the parts, or [N]), times sigmoid
+    or silu (gate_act) of gate_logits [T, N] (may be a column slice). Returns
+    [T, N] in out_dtype."""
+    T, N = o.shape
+    assert o.dtype == torch.float32 and o.is_contiguous() and N % groups == 0
+    assert w.numel() in (N, N // groups) and gate_act in ("sigmoid", "silu")
+    if not o.is_cuda:
+        return torch_ref.gated_rms_norm(o, w, groups, gate_logits, gate_act, eps, out_dtype)
+    lib, hip = _lib()
+    assert w.dtype == torch.float32 and w.is_contiguous()
+    out = torch.empty(T, N, dtype=out_dtype, device=o.device)
+    rc = lib.oa_gated_rms_norm(
+        hip.current_stream_ptr(), o.data_ptr(), w.data_ptr(), w.numel(), gate_logits.data_ptr(),
+        _rows(gate_logits), _dt(gate_logits), 0 if gate_act == "sigmoid" else 1, out.data_ptr(),
+        _dt(out), T, N, groups, float(eps))
+    hip.check(rc, "oa_gated_rms_norm")
     return out
 
 

@@ -435,30 +435,41 @@ def gelu_tanh(z):
 
 
 def act_mul(gate, up, act):
+    """act: "silu" | "gelu_tanh" | ("clamp_swish", limit, alpha):
+    g = min(gate, limit), u = clamp(up, -limit, limit), g sigmoid(alpha g) (u + 1)."""
     g = gate.float()
+    if isinstance(act, tuple):
+        kind, limit, alpha = act
+        assert kind == "clamp_swish"
+        g = g.clamp(max=limit)
+        u = up.float().clamp(-limit, limit)
+        return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gate.dtype)
     a = torch.nn.functional.silu(g) if act == "silu" else gelu_tanh(g)
     return (a * up.float()).to(gate.dtype)
 
 
-def route_topk(logits, correction, top, groups, keep, scale, score):
+def route_topk(logits, correction, top, groups, keep, scale, score, rating="top2",
+               renorm=True):
     """logits float32 [T, E] -> (experts int32 [T, top], weights float32
     [T, top]). Scores are sigmoid or softmax of the logits; the choice uses
     c = score + correction inside the `keep` top-rated of `groups` runs of
-    neighbouring experts (rating: max1(c) + max2(c)); weights
-    w_j = scale * s_j / (sum_k s_k + 1e-20) over the picked experts."""
+    neighbouring experts (rating: max1(c) + max2(c), or max(c) with rating
+    "max"); weights w_j = scale * s_j / (sum_k s_k + 1e-20) over the picked
+    experts, or scale * s_j with renorm off."""
     T, E = logits.shape
     s = torch.sigmoid(logits) if score == "sigmoid" else torch.softmax(logits, -1)
     choice = s + correction.float() if correction is not None else s.clone()
     if groups > 1:
         per = E // groups
-        gs = choice.view(T, groups, per).topk(min(2, per), dim=-1).values.sum(-1)
+        gs = choice.view(T, groups, per).topk(1 if rating == "max" else min(2, per),
+                                              dim=-1).values.sum(-1)
         best = gs.topk(keep, dim=-1).indices
         ok = torch.zeros(T, groups, dtype=torch.bool, device=logits.device)
         ok.scatter_(1, best, True)
         choice = choice.masked_fill(~ok.repeat_interleave(per, dim=1), float("-inf"))
     idx = choice.topk(top, dim=-1).indices
     w = s.gather(1, idx)
-    w = w / (w.sum(-1, keepdim=True) + 1e-20) * scale
+    w = w / (w.sum(-1, keepdim=True) + 1e-20) * scale if renorm else w * scale
     return idx.to(torch.int32), w
 
 
@@ -475,3 +486,104 @@ def moe_pairs_mlp(x, w13, w2, idx, wts, act):
             a = act_mul(gu[:, :inter], gu[:, inter:], act)
             out[t] += wts[t, j] * torch.nn.functional.linear(a, w2[e])[0].float()
     return out.to(x.dtype)
+
+
+# ---------------------------------------------------------------------------
+# Pre-norm decoders with latent attention and decayed linear attention.
+
+
+def add_layer_norm(residual, y, w, eps, out_dtype, y2=None, y2_gate=None):
+    """residual (float32 [T, C], in place) += y + sigmoid(y2_gate) * y2 (each
+    optional; y2_gate [T] scales the rows of y2). With w: returns the layer
+    norm (x - mean) / sqrt(mean((x - mean)^2) + eps) * w of the new residual
+    in out_dtype."""
+    if y is not None:
+        residual += y.float()
+    if y2 is not None:
+        g = torch.sigmoid(y2_gate.float()).unsqueeze(-1) if y2_gate is not None else 1.0
+        residual += g * y2.float()
+    if w is None:
+        return None
+    mu = residual.mean(-1, keepdim=True)
+    d = residual - mu
+    return (d * torch.rsqrt(d.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(out_dtype)
+
+
+def _rotate_pairs(x, pos, inv_freq):
+    """x [T, ..., n] float32: channel pairs (2i, 2i+1), i < len(inv_freq),
+    turn by pos * inv_freq[i]; the rest pass."""
+    n = 2 * inv_freq.numel()
+    ang = pos.float().view(-1, *([1] * (x.dim() - 1))) * inv_freq.float()
+    c, s = torch.cos(ang), torch.sin(ang)
+    u, v = x[..., 0:n:2], x[..., 1:n:2]
+    out = x.clone()
+    out[..., 0:n:2] = u * c - v * s
+    out[..., 1:n:2] = v * c + u * s
+    return out
+
+
+def latent_kv_prepare(dkv, norm_w, inv_freq, rank, rot, eps, k_cache, pos, slot_mapping):
+    """dkv [T, rank + rot]: the first `rank` columns, RMS-normed with norm_w,
+    and the last `rot`, rotated by position, go to the token's cache row
+    [rank + rot]."""
+    x = dkv.float()
+    c = x[:, :rank]
+    c = c * torch.rsqrt(c.pow(2).mean(-1, keepdim=True) + eps) * norm_w.float()
+    kr = _rotate_pairs(x[:, rank:rank + rot], pos, inv_freq)
+    nb, bs = k_cache.shape[0], k_cache.shape[1]
+    k_cache.view(nb * bs, rank + rot)[slot_mapping.long()] = torch.cat([c, kr], -1).to(k_cache.dtype)
+
+
+def latent_q_assemble(q, q_lat, inv_freq, H, D, rot, pos):
+    """q [T, H*(D+rot)] (per head: D unrotated, rot rotated channels), q_lat
+    [H, T, rank] (the unrotated part taken through the key up-projection).
+    Returns [T, H, rank + rot]: q_lat beside the rotated part."""
+    T = q.shape[0]
+    qr = _rotate_pairs(q.float().view(T, H, D + rot)[..., D:], pos, inv_freq)
+    return torch.cat([q_lat.float().transpose(0, 1), qr], -1).to(q.dtype).contiguous()
+
+
+def decay_linear_attention(q, k, v, z, z_bias, inv_tau, head_decay, state, cu, past, slots,
+                           H, D, Dv, act, q_scale):
+    """S_t = diag(a_t) S_{t-1} + k_t v_t^T, o_t = S_t^T q_t per head, continued
+    from `state` [slots, H, Dv, D] float32 (S transposed; zero at position 0
+    whatever the slot holds). a_t = head_decay[h] for every channel, or
+    sigmoid(z_t + z_bias)^(inv_tau) per key channel when z is given. act
+    "silu" is applied to q, k and v first; q is then scaled. Returns the
+    read-out [T, H*Dv] float32; updates state."""
+    T = q.shape[0]
+    f = (lambda t: torch.nn.functional.silu(t.float())) if act == "silu" else (lambda t: t.float())
+    qf = (f(q) * q_scale).view(T, H, D)
+    kf, vf = f(k).view(T, H, D), f(v).view(T, H, Dv)
+    if z is not None:
+        zz = z.float() + z_bias.float()
+        a = torch.exp(torch.nn.functional.logsigmoid(zz) * inv_tau).view(T, H, D)
+    else:
+        a = head_decay.float().view(1, H, 1).expand(T, H, D)
+    out = torch.empty(T, H, Dv, dtype=torch.float32, device=q.device)
+    for bi in range(len(cu) - 1):
+        lo, hi = cu[bi], cu[bi + 1]
+        if hi == lo:
+            continue
+        S = state[slots[bi]].transpose(-1, -2).clone()      # [H, D, Dv]
+        if past[bi] == 0:
+            S.zero_()
+        for t in range(lo, hi):
+            S = S * a[t].unsqueeze(-1) + kf[t].unsqueeze(-1) * vf[t].unsqueeze(1)
+            out[t] = torch.einsum("hdv,hd->hv", S, qf[t])
+        state[slots[bi]] = S.transpose(-1, -2)
+    return out.view(T, H * Dv)
+
+
+def gated_rms_norm(o, w, groups, gate_logits, gate_act, eps, out_dtype):
+    """o [T, N] float32: RMS norm over each of `groups` equal parts, times w
+    ([N/groups], shared by the parts, or [N]), times sigmoid or silu of
+    gate_logits [T, N]."""
+    T, N = o.shape
+    x = o.view(T, groups, N // groups)
+    x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps)
+    wf = w.float()
+    x = (x * wf).view(T, N) if wf.numel() == N // groups else x.reshape(T, N) * wf
+    g = gate_logits.float()
+    g = torch.sigmoid(g) if gate_act == "sigmoid" else torch.nn.functional.silu(g)
+    return (x * g).to(out_dtype)
