@@ -186,3 +186,67 @@ def forward(cfg, W, tokens, layers_out=None):
         if layers_out is not None:
             layers_out.append(x.clone())
     return layer_norm(x, W["final.norm"], eps) @ W["head"].T
+
+
+def greedy(cfg, W, prompt, n):
+    toks = list(prompt)
+    for _ in range(n):
+        toks.append(int(forward(cfg, W, toks)[-1].argmax()))
+    return toks[len(prompt):]
+
+
+def random_weights(cfg, seed=0, decay_rank=5):
+    """Random tensors under the checkpoint's names for a config dictionary."""
+    g = torch.Generator().manual_seed(seed)
+    C, V = cfg["width"], cfg["vocab"]
+    rn = lambda *s, std=1.0: torch.randn(*s, generator=g) * std
+    W = {"embed": rn(V, C, std=0.5), "head": rn(V, C, std=C ** -0.5),
+         "final.norm": 1.0 + 0.2 * rn(C)}
+
+    def ff(prefix, inner):
+        W[prefix + "gate"] = rn(inner, C, std=1.5 * C ** -0.5)
+        W[prefix + "up"] = rn(inner, C, std=1.5 * C ** -0.5)
+        W[prefix + "down"] = rn(C, inner, std=inner ** -0.5)
+
+    for i, layer in enumerate(cfg["layers"]):
+        p, m = f"l{i}.", layer["mixer"]
+        H, D, Dv = m["heads"], m["dim"], m["vdim"]
+        W[p + "norm1"] = 1.0 + 0.2 * rn(C)
+        if layer["type"] == "latent_attention":
+            R, rot = m["kv_rank"], m["rot_dim"]
+            W[p + "mix.q"] = rn(H * (D + rot), C, std=C ** -0.5)
+            if m.get("kv_from") is None:
+                W[p + "mix.dkv"] = rn(R + rot, C, std=C ** -0.5)
+                W[p + "mix.dkv.norm"] = 1.0 + 0.2 * rn(R)
+            W[p + "mix.uk"] = rn(H * D, R, std=R ** -0.5)
+            W[p + "mix.uv"] = rn(H * Dv, R, std=R ** -0.5)
+            W[p + "mix.sink"] = rn(H)
+            W[p + "mix.g"] = rn(H, C, std=C ** -0.5)
+        else:
+            W[p + "mix.q"] = rn(H * D, C, std=C ** -0.5)
+            W[p + "mix.k"] = rn(H * D, C, std=C ** -0.5)
+            W[p + "mix.v"] = rn(H * Dv, C, std=C ** -0.5)
+            W[p + "mix.g"] = rn(H * Dv, C, std=C ** -0.5)
+            if layer["type"] == "gla":
+                W[p + "mix.a1"] = rn(decay_rank, C, std=C ** -0.5)
+                W[p + "mix.a2"] = rn(H * D, decay_rank, std=2.0 * decay_rank ** -0.5)
+                W[p + "mix.a2.b"] = 1.0 + rn(H * D)
+                W[p + "mix.norm"] = 1.0 + 0.2 * rn(Dv)
+            else:
+                W[p + "mix.norm"] = 1.0 + 0.2 * rn(H * Dv)
+        W[p + "mix.o"] = rn(C, H * Dv, std=(H * Dv) ** -0.5)
+        mlp = layer.get("mlp")
+        if mlp is None:
+            continue
+        W[p + "norm2"] = 1.0 + 0.2 * rn(C)
+        if mlp["kind"] == "dense":
+            ff(p + "mlp.", mlp["ff"])
+        else:
+            n = mlp["router"]["experts"]
+            W[p + "mlp.router"] = rn(n, C, std=2.0 * C ** -0.5)
+            for e in range(n):
+                ff(f"{p}mlp.e{e}.", mlp["expert"]["ff"])
+            if mlp.get("shared"):
+                ff(p + "mlp.shared.", mlp["shared"]["ff"])
+                W[p + "mlp.shared.sg"] = rn(1, C, std=C ** -0.5)
+    return W
