@@ -83,11 +83,11 @@ def main() -> None:
     ap.add_argument("--mode", choices=["turn", "multiturn", "concurrent", "layers"],
                     default="turn",
                     help="layers: prefill/decode throughput of the hybrid decoders "
-                         "(Povazen, Vazilorn) beside llama / llama-moe layers of equal "
+                         "(Povazen, Vazilorn, Rafodra) beside llama / llama-moe layers of equal "
                          "size (extra mode; prints one JSON line per size and batch)")
     ap.add_argument("--layer-models", default="llama,povazen",
                     help="layers mode: which models to run (llama, povazen, llama-moe, "
-                         "vazilorn, vazilorn-w512, vazilorn-moe)")
+                         "vazilorn, vazilorn-w512, vazilorn-moe, rafodra, rafodra-moe)")
     ap.add_argument("--layer-sizes", default="", help="layers mode: size names (default all)")
     ap.add_argument("--layer-batches", default="1,8", help="layers mode: batch sizes")
     ap.add_argument("--concurrency", type=int, default=8, help="sessions in concurrent mode")

@@ -265,14 +265,16 @@ class RoutedExperts(nn.Module):
 
         T, C = x.shape
         I, top = self.r.ff, self.r.top
-        if (x.is_cuda and x.dtype == torch.bfloat16 and self.act == "silu"
+        fast_act = self.act == "silu" or (isinstance(self.act, tuple)
+                                          and self.act[0] == "clamp_swish")
+        if (x.is_cuda and x.dtype == torch.bfloat16 and fast_act
                 and C % 16 == 0 and I % 16 == 0 and self.force_path is None):
             # the framework's grouped expert GEMV kernels (pair- or expert-major)
             flat_t = torch.arange(T, device=x.device, dtype=torch.int32).repeat_interleave(top)
             y = ops.moe_grouped_mlp(x.contiguous(), self.w13, None, self.w2, None,
                                     idx.reshape(-1), flat_t.contiguous(),
                                     wts.reshape(-1).contiguous(), I, False,
-                                    num_experts=self.r.experts)
+                                    num_experts=self.r.experts, act=self.act)
             return y.view(T, top, C).float().sum(1).to(x.dtype)
         return mx.moe_pairs_mlp(x.contiguous(), self.w13, self.w2, idx, wts, self.act)
 

@@ -345,6 +345,7 @@ def moe_grouped_mlp(
     i_local: int,
     fp8: bool,
     num_experts: int = 0,
+    act=None,
 ) -> torch.Tensor:
     """Grouped MoE expert MLP (GPU decode path): one gateup launch + one down
     launch for ALL (token, expert) pairs of a layer — no per-expert loop, no
@@ -357,7 +358,15 @@ def moe_grouped_mlp(
       * expert-major (P > OPSAGENT_MOE_EMAJ_MIN_P, needs num_experts): one
         block column per EXPERT; weights stream once per GROUP of 8 matched
         pairs, cutting the weight traffic up to 8x at big decode batches
+    act: None / "silu", or ("clamp_swish", limit, alpha) for the clamped gate
+    g' = min(g, limit), u' = clamp(u, -limit, limit), g' sigmoid(alpha g') (u' + 1).
     """
+    if isinstance(act, tuple):
+        assert act[0] == "clamp_swish"
+        actk, limit, alpha = 2, float(act[1]), float(act[2])
+    else:
+        assert act in (None, "silu")
+        actk, limit, alpha = 0, 0.0, 0.0
     assert x.is_cuda and x.dtype == torch.bfloat16 and x.is_contiguous()
     # stride-0 expand views have a data_ptr that covers ONE element — the
     # kernels index these linearly, so contiguity is load-bearing
@@ -370,27 +379,27 @@ def moe_grouped_mlp(
     H = w2.shape[1]
     emaj_min = int(os.environ.get("OPSAGENT_MOE_EMAJ_MIN_P", "64"))
     use_emaj = num_experts > 0 and P >= emaj_min and P <= 2048
-    act = torch.empty(P, i_local, dtype=x.dtype, device=x.device)
+    mid = torch.empty(P, i_local, dtype=x.dtype, device=x.device)
     if use_emaj:
-        rc = lib.oa_moe_gateup_emaj(
+        rc = lib.oa_moe_gateup_emaj_act(
             hip.current_stream_ptr(), x.data_ptr(), w13.data_ptr(),
             w13_scale.data_ptr() if fp8 else None,
-            expert_ids.data_ptr(), token_ids.data_ptr(), act.data_ptr(),
-            P, num_experts, i_local, K, 1 if fp8 else 0,
+            expert_ids.data_ptr(), token_ids.data_ptr(), mid.data_ptr(),
+            P, num_experts, i_local, K, 1 if fp8 else 0, actk, limit, alpha,
         )
         hip.check(rc, "oa_moe_gateup_emaj")
     else:
-        rc = lib.oa_moe_gateup(
+        rc = lib.oa_moe_gateup_act(
             hip.current_stream_ptr(), x.data_ptr(), w13.data_ptr(),
             w13_scale.data_ptr() if fp8 else None,
-            expert_ids.data_ptr(), token_ids.data_ptr(), act.data_ptr(),
-            P, i_local, K, 1 if fp8 else 0,
+            expert_ids.data_ptr(), token_ids.data_ptr(), mid.data_ptr(),
+            P, i_local, K, 1 if fp8 else 0, actk, limit, alpha,
         )
         hip.check(rc, "oa_moe_gateup")
     y = torch.empty(P, H, dtype=x.dtype, device=x.device)
     if use_emaj:
         rc = lib.oa_moe_down_emaj(
-            hip.current_stream_ptr(), act.data_ptr(), w2.data_ptr(),
+            hip.current_stream_ptr(), mid.data_ptr(), w2.data_ptr(),
             w2_scale.data_ptr() if fp8 else None,
             expert_ids.data_ptr(), pair_weights.data_ptr(), y.data_ptr(),
             P, num_experts, H, i_local, 1 if fp8 else 0,
@@ -398,7 +407,7 @@ def moe_grouped_mlp(
         hip.check(rc, "oa_moe_down_emaj")
     else:
         rc = lib.oa_moe_down(
-            hip.current_stream_ptr(), act.data_ptr(), w2.data_ptr(),
+            hip.current_stream_ptr(), mid.data_ptr(), w2.data_ptr(),
             w2_scale.data_ptr() if fp8 else None,
             expert_ids.data_ptr(), pair_weights.data_ptr(), y.data_ptr(),
             P, H, i_local, 1 if fp8 else 0,

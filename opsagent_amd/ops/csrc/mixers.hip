@@ -597,7 +597,13 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
     const int* __restrict__ cu, const int* __restrict__ past,
     const int* __restrict__ block_table, int max_blocks, int block_size,
     const float* __restrict__ slopes, const float* __restrict__ sinks, int B, int H, int G,
-    int D, int Dv, int HB, float scale, int nsplit, int window, int64_t vrow) {
+    int D, int Dv, int HB, float scale, int nsplit, int window, int vrow, int hrows) {
+    // hrows (decode steps of many query heads per kv head): a step brings one
+    // token per sequence, so the 16 columns of a wave's tile are 16 HEADS at
+    // that token's position instead of 16 tokens of one head; a block covers
+    // 64 heads of one kv head and every staged key/value tile serves them
+    // all. The head (and with it slope, sink, gate and output row) is then a
+    // per-lane value.
     // NT: 16-token sub-tiles per wave. Every K and V fragment read from LDS
     // feeds NT MFMAs, and a staged tile serves NT times the query rows.
     extern __shared__ float lds[];
@@ -609,9 +615,12 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
     const int TT = 4 / HB, TQ = 16 * TT * NT;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lc = lane & 15, lg = lane >> 4;
-    const int hgroups = R / HB;
+    const int hgroups = hrows ? (R + 63) / 64 : R / HB;
     const int g = blockIdx.y / hgroups;
-    const int h = g * R + (blockIdx.y % hgroups) * HB + wave % HB;
+    const int hoff = (blockIdx.y % hgroups) * 64 + wave * 16;      // hrows: the wave's first head
+    const int h = hrows ? g * R + min(hoff + lc, R - 1)
+                        : g * R + (blockIdx.y % hgroups) * HB + wave % HB;
+    const int hvalid = max(0, min(16, R - hoff));                  // hrows: heads in this wave
     const int split = blockIdx.z;
     int tile = blockIdx.x, b = 0, lo = 0, n = 0;
     for (; b < B; ++b) {
@@ -623,14 +632,18 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
     }
     if (b >= B) return;
     const int pb = past[b];
-    const int t0 = tile * TQ + (wave / HB) * 16 * NT;   // this wave's first local token
+    const int t0 = hrows ? 0 : tile * TQ + (wave / HB) * 16 * NT;   // this wave's first local token
     int ntok[NT], pos[NT];
 #pragma unroll
     for (int u = 0; u < NT; ++u) {
         ntok[u] = max(0, min(16, n - (t0 + 16 * u)));
         pos[u] = pb + t0 + 16 * u + lc;                  // this lane's token position
+        if (hrows) {
+            ntok[u] = (u == 0 && n > 0) ? hvalid : 0;    // valid columns = valid heads
+            pos[u] = pb;
+        }
     }
-    const int wave_ntok = max(0, min(16 * NT, n - t0));
+    const int wave_ntok = hrows ? ((n > 0 && hvalid > 0) ? 1 : 0) : max(0, min(16 * NT, n - t0));
     const int wave_last = pb + t0 + wave_ntok - 1;
     const int block_last = pb + min(n, tile * TQ + TQ) - 1;
     const int* bt = block_table + (int64_t)b * max_blocks;
@@ -645,7 +658,7 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
     s8_t qf8[NT][QK32 ? MAXD / 2 : 1];
 #pragma unroll
     for (int u = 0; u < NT; ++u) {
-        const int tk = lo + t0 + 16 * u + min(lc, max(ntok[u] - 1, 0));
+        const int tk = hrows ? lo : lo + t0 + 16 * u + min(lc, max(ntok[u] - 1, 0));
         const bf16s* qr = q + ((int64_t)min(tk, lo + n - 1) * H + h) * D;
         if (QK32) {
 #pragma unroll
@@ -698,7 +711,7 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
         const int64_t sk_ = okk ? ((int64_t)bt[keyk >> bsh] << bsh) + (keyk & bmask) : 0;
         const int64_t sv_ = okv ? ((int64_t)bt[keyv >> bsh] << bsh) + (keyv & bmask) : 0;
         const bf16s* kp = k_cache + (sk_ * G + g) * D;
-        const bf16s* vp = v_cache + sv_ * vrow + g * Dv;
+        const bf16s* vp = v_cache + (sv_ * vrow + g * Dv);
 #pragma unroll
         for (int u = 0; u < KC; ++u) {
             const int c = kc0 + 4 * u;
@@ -845,7 +858,7 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
 #pragma unroll
     for (int u = 0; u < NT; ++u) {
         if (lc >= ntok[u]) continue;
-        const int tok = lo + t0 + 16 * u + lc;
+        const int tok = hrows ? lo : lo + t0 + 16 * u + lc;
         if (nsplit == 1) {
             const float lt = sinks ? l[u] + __builtin_amdgcn_exp2f(sinks[h] * LOG2E - m[u]) : l[u];
             const float gt = (gate ? sigmoidf_(ldf(gate, (int64_t)tok * gs + h)) : 1.0f) / lt;
@@ -1353,7 +1366,10 @@ extern "C" int oa_attn_prepare(void* stream, const void* qkv, int64_t qs, const 
 // bytes. path 1 = matrix cores (bf16, sizes multiples of 16), 0 = VALU.
 static int attn_path(int H, int G, int D, int Dv, int dt) {
     if (std::getenv("OPSAGENT_ATTN_VALU")) return 0;
-    return (dt == 0 && D % 16 == 0 && Dv % 16 == 0 && D <= 256 && Dv <= 256) ? 1 : 0;
+    // key sizes above 128 take the matrix-core kernel only in steps of 32:
+    // the 16-wide K step would hold twice the query fragments and spill
+    return (dt == 0 && D % 16 == 0 && Dv % 16 == 0 && D <= 256 && Dv <= 256 &&
+            (D <= 128 || D % 32 == 0)) ? 1 : 0;
 }
 static int attn_hb(int R) { return R % 4 == 0 ? 4 : (R % 2 == 0 ? 2 : 1); }
 
@@ -1399,7 +1415,8 @@ static void launch_attn_mfma(hipStream_t s, dim3 grid, int lds_bytes, const void
                              void* part_o, void* part_ml, const void* cu, const void* past,
                              const void* block_table, int max_blocks, int block_size,
                              const void* slopes, const void* sinks, int B, int H, int G, int D,
-                             int Dv, int HB, float scale, int nsplit, int window, int64_t vrow) {
+                             int Dv, int HB, float scale, int nsplit, int window, int64_t vrow,
+                             int hrows) {
     if (lds_bytes > 48 * 1024)
         (void)hipFuncSetAttribute((const void*)attn_bias_mfma_kernel<MAXD, MAXDV, QK32, NT>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
@@ -1408,7 +1425,7 @@ static void launch_attn_mfma(hipStream_t s, dim3 grid, int lds_bytes, const void
                        (const bf16s*)v_cache, (bf16s*)out, (float*)part_o, (float*)part_ml,
                        (const int*)cu, (const int*)past, (const int*)block_table, max_blocks,
                        block_size, (const float*)slopes, (const float*)sinks, B, H, G, D, Dv, HB,
-                       scale, nsplit, window, vrow);
+                       scale, nsplit, window, (int)vrow, hrows);
 }
 
 // ntiles = sum_b ceil(n_b / TQ) (host-computed). part_* may be null when nsplit == 1.
@@ -1433,10 +1450,13 @@ extern "C" int oa_attn_bias_paged(void* stream, const void* q, const void* gate,
     if (attn_path(H, G, D, Dv, dt)) {
         if (vrow % 8 != 0) return -107;   // 16-byte value loads
         const int R = H / G, HB = attn_hb(R);
-        dim3 grid(ntiles, G * (R / HB), nsplit);
+        // decode steps of 16 or more query heads per kv head put the heads
+        // in the tile's columns
+        const int hrows = (max_chunk == 1 && R >= 16) ? 1 : 0;
+        dim3 grid(ntiles, hrows ? G * CEIL_DIV(R, 64) : G * (R / HB), nsplit);
 #define MF_ARGS                                                                                   \
     s, grid, lds_bytes, q, gate, gs, k_cache, v_cache, out, part_o, part_ml, cu, past, block_table, \
-        max_blocks, block_size, slopes, sinks, B, H, G, D, Dv, HB, scale, nsplit, window, vrow
+        max_blocks, block_size, slopes, sinks, B, H, G, D, Dv, HB, scale, nsplit, window, vrow, hrows
 #define MF(A, Bv)                                                               \
     do {                                                                        \
         if (D % 32 == 0) launch_attn_mfma<A, Bv, true, 1>(MF_ARGS);             \
@@ -1449,9 +1469,9 @@ extern "C" int oa_attn_bias_paged(void* stream, const void* q, const void* gate,
         else if (a == 8 && bv == 4) MF(8, 4);
         else if (a == 8 && bv == 8) MF(8, 8);
         else if (a == 8) MF(8, 16);
-        else if (bv == 4) MF(16, 4);
-        else if (bv == 8) MF(16, 8);
-        else MF(16, 16);
+        else if (bv == 4) launch_attn_mfma<16, 4, true, 1>(MF_ARGS);
+        else if (bv == 8) launch_attn_mfma<16, 8, true, 1>(MF_ARGS);
+        else launch_attn_mfma<16, 16, true, 1>(MF_ARGS);
 #undef MF
 #undef MF_ARGS
         HIP_CHECK_LAUNCH();

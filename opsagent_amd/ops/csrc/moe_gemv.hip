@@ -62,6 +62,17 @@ __device__ __forceinline__ float dot_fp8(const uint32_t* wrow, const uint32_t* x
     return wave_reduce_sum(acc);
 }
 
+// gate activation times up: act 0 silu(g) * u; act 2 the clamped form
+// g' = min(g, limit), u' = clamp(u, -limit, limit), g' sigmoid(alpha g') (u' + 1)
+__device__ __forceinline__ float moe_gate_act(float g, float u, int act, float limit, float alpha) {
+    if (act == 2) {
+        g = fminf(g, limit);
+        u = fminf(fmaxf(u, -limit), limit);
+        return g / (1.0f + __expf(-alpha * g)) * (u + 1.0f);
+    }
+    return g / (1.0f + __expf(-g)) * u;
+}
+
 // ---- gate-up + SiLU ---------------------------------------------------------
 template <bool FP8>
 __global__ __launch_bounds__(256) void moe_gateup_kernel(
@@ -71,7 +82,7 @@ __global__ __launch_bounds__(256) void moe_gateup_kernel(
     const int* __restrict__ expert_ids,   // [P]
     const int* __restrict__ token_ids,    // [P]
     uint32_t* __restrict__ act,           // [P, I] bf16
-    int I, int K) {
+    int I, int K, int actk, float limit, float alpha) {
     const int p = blockIdx.y;
     const int e = expert_ids[p];
     const int lane = threadIdx.x & (WAVE - 1);
@@ -92,7 +103,7 @@ __global__ __launch_bounds__(256) void moe_gateup_kernel(
             u = dot_bf16(wbase + (size_t)(I + row) * wwords, xrow, wwords, lane);
         }
         if (lane == 0) {
-            const float a = g / (1.0f + __expf(-g)) * u;
+            const float a = moe_gate_act(g, u, actk, limit, alpha);
             reinterpret_cast<uint16_t*>(act)[(size_t)p * I + row] = f32_to_bf16(a);
         }
     }
@@ -148,7 +159,7 @@ __global__ __launch_bounds__(256) void moe_emaj_kernel(
     const int* __restrict__ token_ids,    // [P] (GATEUP; ignored for down)
     const float* __restrict__ pair_w,     // [P] (down; ignored for gateup)
     uint32_t* __restrict__ out,           // [P, I] or [P, H] bf16
-    int P, int NROWS /* I or H */, int K) {
+    int P, int NROWS /* I or H */, int K, int actk, float limit, float alpha) {
     const int e = blockIdx.y;
     const int lane = threadIdx.x & (WAVE - 1);
     const int wid = threadIdx.x / WAVE;
@@ -247,7 +258,7 @@ __global__ __launch_bounds__(256) void moe_emaj_kernel(
                             g *= sbase[row];
                             u *= sbase[NROWS + row];
                         }
-                        const float a = g / (1.0f + __expf(-g)) * u;
+                        const float a = moe_gate_act(g, u, actk, limit, alpha);
                         reinterpret_cast<uint16_t*>(out)[(size_t)p * NROWS + row] =
                             f32_to_bf16(a);
                     } else {
@@ -261,10 +272,11 @@ __global__ __launch_bounds__(256) void moe_emaj_kernel(
     }
 }
 
-extern "C" int oa_moe_gateup_emaj(void* stream, const void* x, const void* w,
+extern "C" int oa_moe_gateup_emaj_act(void* stream, const void* x, const void* w,
                                   const void* wscale, const void* expert_ids,
                                   const void* token_ids, void* act, int P,
-                                  int E, int I, int K, int fp8) {
+                                  int E, int I, int K, int fp8, int actk, float limit,
+                                      float alpha) {
     if (K % 16 != 0 || P > EMAJ_MAXP) return -100;
     dim3 grid(min(64, CEIL_DIV(I, 4)), E), block(256);
     if (fp8)
@@ -272,15 +284,23 @@ extern "C" int oa_moe_gateup_emaj(void* stream, const void* x, const void* w,
                            (hipStream_t)stream, (const uint32_t*)x,
                            (const uint32_t*)w, (const float*)wscale,
                            (const int*)expert_ids, (const int*)token_ids,
-                           (const float*)nullptr, (uint32_t*)act, P, I, K);
+                           (const float*)nullptr, (uint32_t*)act, P, I, K, actk, limit, alpha);
     else
         hipLaunchKernelGGL((moe_emaj_kernel<false, true>), grid, block, 0,
                            (hipStream_t)stream, (const uint32_t*)x,
                            (const uint32_t*)w, (const float*)wscale,
                            (const int*)expert_ids, (const int*)token_ids,
-                           (const float*)nullptr, (uint32_t*)act, P, I, K);
+                           (const float*)nullptr, (uint32_t*)act, P, I, K, actk, limit, alpha);
     HIP_CHECK_LAUNCH();
     return 0;
+}
+
+extern "C" int oa_moe_gateup_emaj(void* stream, const void* x, const void* w,
+                                  const void* wscale, const void* expert_ids,
+                                  const void* token_ids, void* act, int P,
+                                  int E, int I, int K, int fp8) {
+    return oa_moe_gateup_emaj_act(stream, x, w, wscale, expert_ids, token_ids, act, P, E, I, K,
+                                  fp8, 0, 0.0f, 0.0f);
 }
 
 extern "C" int oa_moe_down_emaj(void* stream, const void* act, const void* w,
@@ -294,13 +314,35 @@ extern "C" int oa_moe_down_emaj(void* stream, const void* act, const void* w,
                            (hipStream_t)stream, (const uint32_t*)act,
                            (const uint32_t*)w, (const float*)wscale,
                            (const int*)expert_ids, (const int*)nullptr,
-                           (const float*)pair_w, (uint32_t*)y, P, H, I);
+                           (const float*)pair_w, (uint32_t*)y, P, H, I, 0, 0.0f, 0.0f);
     else
         hipLaunchKernelGGL((moe_emaj_kernel<false, false>), grid, block, 0,
                            (hipStream_t)stream, (const uint32_t*)act,
                            (const uint32_t*)w, (const float*)wscale,
                            (const int*)expert_ids, (const int*)nullptr,
-                           (const float*)pair_w, (uint32_t*)y, P, H, I);
+                           (const float*)pair_w, (uint32_t*)y, P, H, I, 0, 0.0f, 0.0f);
+    HIP_CHECK_LAUNCH();
+    return 0;
+}
+
+extern "C" int oa_moe_gateup_act(void* stream, const void* x, const void* w,
+                             const void* wscale, const void* expert_ids,
+                             const void* token_ids, void* act, int P, int I,
+                             int K, int fp8, int actk, float limit, float alpha) {
+    if (K % 16 != 0) return -100;
+    dim3 grid(min(512, CEIL_DIV(I, 4)), P), block(256);
+    if (fp8)
+        hipLaunchKernelGGL((moe_gateup_kernel<true>), grid, block, 0,
+                           (hipStream_t)stream, (const uint32_t*)x,
+                           (const uint32_t*)w, (const float*)wscale,
+                           (const int*)expert_ids, (const int*)token_ids,
+                           (uint32_t*)act, I, K, actk, limit, alpha);
+    else
+        hipLaunchKernelGGL((moe_gateup_kernel<false>), grid, block, 0,
+                           (hipStream_t)stream, (const uint32_t*)x,
+                           (const uint32_t*)w, (const float*)wscale,
+                           (const int*)expert_ids, (const int*)token_ids,
+                           (uint32_t*)act, I, K, actk, limit, alpha);
     HIP_CHECK_LAUNCH();
     return 0;
 }
@@ -309,22 +351,8 @@ extern "C" int oa_moe_gateup(void* stream, const void* x, const void* w,
                              const void* wscale, const void* expert_ids,
                              const void* token_ids, void* act, int P, int I,
                              int K, int fp8) {
-    if (K % 16 != 0) return -100;
-    dim3 grid(min(512, CEIL_DIV(I, 4)), P), block(256);
-    if (fp8)
-        hipLaunchKernelGGL((moe_gateup_kernel<true>), grid, block, 0,
-                           (hipStream_t)stream, (const uint32_t*)x,
-                           (const uint32_t*)w, (const float*)wscale,
-                           (const int*)expert_ids, (const int*)token_ids,
-                           (uint32_t*)act, I, K);
-    else
-        hipLaunchKernelGGL((moe_gateup_kernel<false>), grid, block, 0,
-                           (hipStream_t)stream, (const uint32_t*)x,
-                           (const uint32_t*)w, (const float*)wscale,
-                           (const int*)expert_ids, (const int*)token_ids,
-                           (uint32_t*)act, I, K);
-    HIP_CHECK_LAUNCH();
-    return 0;
+    return oa_moe_gateup_act(stream, x, w, wscale, expert_ids, token_ids, act, P, I, K, fp8, 0,
+                             0.0f, 0.0f);
 }
 
 extern "C" int oa_moe_down(void* stream, const void* act, const void* w,

@@ -82,6 +82,10 @@ def _declare(lib: ctypes.CDLL) -> None:
     lib.oa_moe_down.restype = i
     lib.oa_moe_gateup_emaj.argtypes = [p, p, p, p, p, p, p, i, i, i, i, i]
     lib.oa_moe_gateup_emaj.restype = i
+    lib.oa_moe_gateup_act.argtypes = [p, p, p, p, p, p, p, i, i, i, i, i, f, f]
+    lib.oa_moe_gateup_act.restype = i
+    lib.oa_moe_gateup_emaj_act.argtypes = [p, p, p, p, p, p, p, i, i, i, i, i, i, f, f]
+    lib.oa_moe_gateup_emaj_act.restype = i
     lib.oa_moe_down_emaj.argtypes = [p, p, p, p, p, p, p, i, i, i, i, i]
     lib.oa_moe_down_emaj.restype = i
 

@@ -232,6 +232,16 @@ def attention_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     nsplit = 1
     if ntiles * G < 256 and nkt >= 8:
         nsplit = int(min(nkt // 4, max(1, 512 // max(1, ntiles * G)), 64))
+    # decode steps of many query heads per kv head run one block per 64 heads
+    # (the heads share each staged tile): fewer blocks, so finer key splits
+    if (sb.max_chunk == 1 and H // G >= 16 and dt == 0 and D % 16 == 0 and Dv % 16 == 0
+            and D <= 256 and Dv <= 256 and (D <= 128 or D % 32 == 0) and nkt >= 4):
+        blocks = ntiles * G * ((H // G + 63) // 64)
+        if blocks < 256:
+            # at most 16: a captured step sizes nkt for the longest context
+            # the pool allows, and merging many (mostly empty) partials costs
+            # more than the splits save
+            nsplit = int(min(nkt // 2, max(1, 512 // blocks), 16))
     out = torch.empty(T, H * Dv, dtype=q.dtype, device=q.device)
     part_o = part_ml = None
     if nsplit > 1:
@@ -615,6 +625,14 @@ def decay_linear_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
     if sb.max_chunk >= 64 and pairs < 192:
         for c in (8, 4, 2):
             if Dv % (4 * c) == 0 and Dv // c >= 16 and pairs * c <= 512:
+                csplit = c
+                break
+    if Dv // csplit > 256 or (D > 128 and Dv // csplit > 64):
+        # at most 256 columns per block; 256-row columns: more than 64 per
+        # block would hold two or four per lane pass and spill registers
+        cap = 64 if D > 128 else 256
+        for c in range(csplit, Dv + 1):
+            if Dv % c == 0 and Dv // c <= cap:
                 csplit = c
                 break
     rc = lib.oa_decay_scan(

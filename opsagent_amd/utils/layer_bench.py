@@ -20,6 +20,8 @@ from opsagent_amd.engine.config import (
     ModelSpec,
     povazen_config_dict,
     povazen_spec_from_dict,
+    rafodra_config_dict,
+    rafodra_spec_from_dict,
     vazilorn_config_dict,
     vazilorn_spec_from_dict,
 )
@@ -60,8 +62,24 @@ def specs_for(size) -> Dict[str, object]:
             name=f"vazilorn-{tag}-{name}",
         )
 
+    def rf(pattern, tag):
+        # every mixer kind once per four layers: lightning, gated linear
+        # attention, latent attention, latent attention on the same latent.
+        # Linear-attention heads have llama's head size; the cached latent is
+        # 192 + 64 wide (one row per token for all heads)
+        return rafodra_spec_from_dict(
+            rafodra_config_dict(vocab=32000, width=width, pattern=(pattern * layers)[:2 * layers],
+                                heads=heads, dim=dim, vdim=dim, ff=ff, kv_rank=192, rot_dim=64,
+                                rot_base=500000.0, lin_heads=heads, lin_dim=dim, lin_vdim=dim,
+                                experts=experts, top=top, expert_ff=eff, groups=4, keep=2,
+                                router_scale=2.0, limit=7.0, shared_ff=eff, shared_limit=7.0,
+                                embed_scale=1.0),
+            name=f"rafodra-{tag}-{name}",
+        )
+
     return {
         "llama": llama, "povazen": hybrid, "llama-moe": llama_moe,
+        "rafodra": rf("LdGdAdSd", "dense"), "rafodra-moe": rf("LmGmAmSm", "moe"),
         # a window wider than the prompt: the attention kernels do llama's work
         "vazilorn": vz("d", 8192, "dense"),
         # a window that pays: keys beyond it are never read
@@ -72,7 +90,7 @@ def specs_for(size) -> Dict[str, object]:
 
 # which model each one is measured against
 BASELINE_OF = {"povazen": "llama", "vazilorn": "llama", "vazilorn-w512": "llama",
-               "vazilorn-moe": "llama-moe"}
+               "vazilorn-moe": "llama-moe", "rafodra": "povazen", "rafodra-moe": "vazilorn-moe"}
 
 
 def _run(spec, batch: int, prompt: int, decode: int, reps: int) -> Dict[str, float]:

@@ -26,9 +26,13 @@ FILES = ["gemv.hip", "attention_prefill.hip", "attention_decode.hip", "fp8_moe.h
 # columns per block (two or four columns per lane pass at 1024 threads); the
 # dispatch splits such heads over blocks instead (one column per pass, no
 # spill), so these instantiations only serve value sizes that do not divide.
+# decay_scan_kernel<16, 2|4>: the same geometry in the decayed linear
+# attention recurrence, and the same dispatch rule.
 ALLOWED_SCRATCH = {"gemm_fp8_kernel_v2ILb0E": 80,
                    "delta_fused_kernelILi16ELi2E": 16,
-                   "delta_fused_kernelILi16ELi4E": 192}
+                   "delta_fused_kernelILi16ELi4E": 192,
+                   "decay_scan_kernelILi16ELi2E": 12,
+                   "decay_scan_kernelILi16ELi4E": 200}
 
 
 @pytest.mark.skipif(shutil.which("hipcc") is None, reason="hipcc not on PATH")

@@ -214,7 +214,9 @@ PORTIONS = ([150], [5, 2, 9, 1, 1, 16, 3, 40, 8, 65], [140] + [1] * 10)
 
 @pytest.mark.parametrize("mode", MODES)
 @pytest.mark.parametrize("geom", [(3, 12, 10, 18, 6), (4, 16, 16, 32, 16), (5, 8, 24, 40, 8),
-                                  (2, 32, 32, 96, 32), (6, 16, 8, 20, 4)])
+                                  (2, 32, 32, 96, 32), (6, 16, 8, 20, 4),
+                                  # 16 and more heads: decoded tokens put the heads in the tile
+                                  (16, 16, 16, 32, 16), (20, 16, 32, 48, 16), (72, 16, 16, 16, 16)])
 def test_latent_attention_alone(mode, geom):
     """The mixer on a given input through the paged cache: one portion, uneven
     portions, token by token at the end; then a second layer's queries on
@@ -290,7 +292,8 @@ def test_sink_takes_weight(mode):
 
 @pytest.mark.parametrize("mode", MODES)
 @pytest.mark.parametrize("kind", ["L", "G"])
-@pytest.mark.parametrize("geom", [(2, 20, 12), (4, 32, 32), (3, 7, 5), (1, 64, 128), (2, 130, 36)])
+@pytest.mark.parametrize("geom", [(2, 20, 12), (4, 32, 32), (3, 7, 5), (1, 64, 128), (2, 130, 36),
+                                  (1, 160, 96), (1, 16, 320)])
 def test_linear_attention_alone(mode, kind, geom):
     """Lightning and gated linear attention on a given input: the state slot
     carries the recurrence over portions of any size; a used slot starts
