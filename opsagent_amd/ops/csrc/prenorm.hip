@@ -15,68 +15,129 @@
 //                                              one float32 logit per token)
 //   residual = r                              (if anything was added)
 //   out = (r - mean(r)) / sqrt(mean((r - mean(r))^2) + eps) * w   (if w)
-// One block per token. The first 256 * LN_NR channels of the row stay in
-// registers between the passes; wider rows re-read the (just written)
+// One block per token, 16 bytes per lane and access where the row allows.
+// The first 256 * LN_NR channels of the row stay in registers between the
+// passes; wider rows re-read the (just written)
 // residual for the rest. The variance is the mean of squared deviations
 // from the already known mean: two passes, no cancellation.
 #define LN_NR 16
 
-template <typename TC>
+__device__ __forceinline__ void ld4(const float* p, int64_t i, float* o) {
+    const float4 a = *reinterpret_cast<const float4*>(p + i);
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+}
+__device__ __forceinline__ void ld4(const bf16s* p, int64_t i, float* o) {
+    const uint2 a = *reinterpret_cast<const uint2*>(p + i);
+    o[0] = bf16_lo(a.x); o[1] = bf16_hi(a.x); o[2] = bf16_lo(a.y); o[3] = bf16_hi(a.y);
+}
+__device__ __forceinline__ void st4(float* p, int64_t i, const float* v) {
+    *reinterpret_cast<float4*>(p + i) = make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void st4(bf16s* p, int64_t i, const float* v) {
+    uint2 a;
+    a.x = pack_bf16x2(v[0], v[1]);
+    a.y = pack_bf16x2(v[2], v[3]);
+    *reinterpret_cast<uint2*>(p + i) = a;
+}
+
+// VEC: a thread takes 4 consecutive channels at a time (C % 4 == 0, rows and
+// bases aligned to 4 elements); otherwise one channel at a time.
+template <typename TC, bool VEC>
 __global__ __launch_bounds__(256) void add_layer_norm_kernel(
     float* __restrict__ residual, const TC* __restrict__ y, int64_t ys,
     const TC* __restrict__ y2, int64_t y2s, const float* __restrict__ g2, int64_t g2s,
     const float* __restrict__ w, TC* __restrict__ out, int C, float eps) {
     __shared__ float red_a[16], red_b[16];
+    constexpr int W = VEC ? 4 : 1;            // channels per step
+    constexpr int NS = LN_NR / W;             // steps kept in registers
     const int t = blockIdx.x, tid = threadIdx.x;
     float* r = residual + (int64_t)t * C;
     const TC* yr = y ? y + (int64_t)t * ys : nullptr;
     const TC* y2r = y2 ? y2 + (int64_t)t * y2s : nullptr;
     const float gate = (y2 && g2) ? sigmoidf_(g2[(int64_t)t * g2s]) : 1.0f;
     const bool adds = y || y2;
+    // channel of step j, element e: (tid + 256 j) * W + e
+    auto load = [&](int c, float* x) {
+        if (VEC) {
+            ld4(r, c, x);
+            float a[4];
+            if (yr) {
+                ld4(yr, c, a);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) x[e] += a[e];
+            }
+            if (y2r) {
+                ld4(y2r, c, a);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) x[e] += gate * a[e];
+            }
+            if (adds) st4(r, c, x);
+        } else {
+            x[0] = r[c];
+            if (yr) x[0] += ldf(yr, c);
+            if (y2r) x[0] += gate * ldf(y2r, c);
+            if (adds) r[c] = x[0];
+        }
+    };
     float vals[LN_NR];
     float sum = 0.0f;
 #pragma unroll
-    for (int j = 0; j < LN_NR; ++j) {
-        const int c = tid + 256 * j;
-        float x = 0.0f;
-        if (c < C) {
-            x = r[c];
-            if (yr) x += ldf(yr, c);
-            if (y2r) x += gate * ldf(y2r, c);
-            if (adds) r[c] = x;
-        }
-        vals[j] = x;
-        sum += x;
+    for (int j = 0; j < NS; ++j) {
+        const int c = (tid + 256 * j) * W;
+#pragma unroll
+        for (int e = 0; e < W; ++e) vals[j * W + e] = 0.0f;
+        if (c < C) load(c, vals + j * W);
+#pragma unroll
+        for (int e = 0; e < W; ++e) sum += vals[j * W + e];
     }
-    for (int c = tid + 256 * LN_NR; c < C; c += 256) {
-        float x = r[c];
-        if (yr) x += ldf(yr, c);
-        if (y2r) x += gate * ldf(y2r, c);
-        if (adds) r[c] = x;
-        sum += x;
+    for (int c = (tid + 256 * NS) * W; c < C; c += 256 * W) {
+        float x[W];
+        load(c, x);
+#pragma unroll
+        for (int e = 0; e < W; ++e) sum += x[e];
     }
     if (!w) return;
     const float mean = block_reduce_sum<4>(sum, red_a) / (float)C;
     float sq = 0.0f;
 #pragma unroll
-    for (int j = 0; j < LN_NR; ++j) {
-        const int c = tid + 256 * j;
-        const float d = vals[j] - mean;
-        if (c < C) sq += d * d;
+    for (int j = 0; j < NS; ++j) {
+        const int c = (tid + 256 * j) * W;
+        if (c < C) {
+#pragma unroll
+            for (int e = 0; e < W; ++e) {
+                const float d = vals[j * W + e] - mean;
+                sq += d * d;
+            }
+        }
     }
-    for (int c = tid + 256 * LN_NR; c < C; c += 256) {
-        const float d = r[c] - mean;
-        sq += d * d;
+    for (int c = (tid + 256 * NS) * W; c < C; c += 256 * W) {
+#pragma unroll
+        for (int e = 0; e < W; ++e) {
+            const float d = r[c + e] - mean;
+            sq += d * d;
+        }
     }
     const float var = block_reduce_sum<4>(sq, red_b) / (float)C;
     const float rs = 1.0f / sqrtf(var + eps);
     TC* o = out + (int64_t)t * C;
 #pragma unroll
-    for (int j = 0; j < LN_NR; ++j) {
-        const int c = tid + 256 * j;
-        if (c < C) stf(o, c, (vals[j] - mean) * rs * w[c]);
+    for (int j = 0; j < NS; ++j) {
+        const int c = (tid + 256 * j) * W;
+        if (c < C) {
+            float x[W];
+#pragma unroll
+            for (int e = 0; e < W; ++e) x[e] = (vals[j * W + e] - mean) * rs * w[c + e];
+            if (VEC) st4(o, c, x);
+            else stf(o, c, x[0]);
+        }
     }
-    for (int c = tid + 256 * LN_NR; c < C; c += 256) stf(o, c, (r[c] - mean) * rs * w[c]);
+    for (int c = (tid + 256 * NS) * W; c < C; c += 256 * W) {
+        float x[W];
+#pragma unroll
+        for (int e = 0; e < W; ++e) x[e] = (r[c + e] - mean) * rs * w[c + e];
+        if (VEC) st4(o, c, x);
+        else stf(o, c, x[0]);
+    }
 }
 
 // y, y2 and out share the activation type dt.
@@ -98,14 +159,24 @@ extern "C" int oa_add_layer_norm(void* stream, void* residual, const void* y, in
     }
     if (dt < 0) return 0;   // nothing to add, nothing to norm
     hipStream_t s = (hipStream_t)stream;
-    if (dt == 1)
-        hipLaunchKernelGGL((add_layer_norm_kernel<float>), dim3(T), dim3(256), 0, s, (float*)residual,
-                           (const float*)y, ys, (const float*)y2, y2s, (const float*)g2, g2s,
-                           (const float*)w, (float*)out, C, eps);
-    else
-        hipLaunchKernelGGL((add_layer_norm_kernel<bf16s>), dim3(T), dim3(256), 0, s, (float*)residual,
-                           (const bf16s*)y, ys, (const bf16s*)y2, y2s, (const float*)g2, g2s,
-                           (const float*)w, (bf16s*)out, C, eps);
+    const int esz = dt == 1 ? 4 : 2;
+    auto al = [&](const void* p, int64_t stride) {
+        return !p || ((uintptr_t)p % (4 * esz) == 0 && stride % 4 == 0);
+    };
+    const bool vec = C % 4 == 0 && (uintptr_t)residual % 16 == 0 && al(y, ys) && al(y2, y2s) &&
+                     al(out, 0) && (!w || (uintptr_t)w % 16 == 0);
+#define LN_LAUNCH(TC, V)                                                                         \
+    hipLaunchKernelGGL((add_layer_norm_kernel<TC, V>), dim3(T), dim3(256), 0, s, (float*)residual, \
+                       (const TC*)y, ys, (const TC*)y2, y2s, (const float*)g2, g2s,               \
+                       (const float*)w, (TC*)out, C, eps)
+    if (dt == 1) {
+        if (vec) LN_LAUNCH(float, true);
+        else LN_LAUNCH(float, false);
+    } else {
+        if (vec) LN_LAUNCH(bf16s, true);
+        else LN_LAUNCH(bf16s, false);
+    }
+#undef LN_LAUNCH
     HIP_CHECK_LAUNCH();
     return 0;
 }

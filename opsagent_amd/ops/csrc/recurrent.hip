@@ -235,44 +235,95 @@ extern "C" int oa_decay_scan(void* stream, const void* q, int64_t qs, const void
 // Gated RMS norm of a float32 read-out o [T, N]: the row is cut into `groups`
 // equal parts, each divided by sqrt(mean(part^2) + eps), times the float32
 // weight (wlen = N: one per channel; wlen = N / groups: shared by the parts),
-// times gate_act(gate): 0 sigmoid, 1 silu. One block per token, a wave per
-// part (one part: the whole block reduces it).
-template <typename TG, typename TO>
+// times gate_act(gate): 0 sigmoid, 1 silu. grid = (tokens, part groups): one
+// part, the whole block reduces the row; several, a wave per part and four
+// parts per block. A lane keeps its channels in registers between the sum
+// and the scaling (GN_NR per lane, the rest is read again).
+#define GN_NR 16
+
+__device__ __forceinline__ float gate_fn(float g, int gate_act) {
+    return gate_act ? g / (1.0f + expf(-g)) : sigmoidf_(g);
+}
+__device__ __forceinline__ void gn_ld4(const float* p, int64_t i, float* o) {
+    const float4 a = *reinterpret_cast<const float4*>(p + i);
+    o[0] = a.x; o[1] = a.y; o[2] = a.z; o[3] = a.w;
+}
+__device__ __forceinline__ void gn_ld4(const bf16s* p, int64_t i, float* o) {
+    const uint2 a = *reinterpret_cast<const uint2*>(p + i);
+    o[0] = bf16_lo(a.x); o[1] = bf16_hi(a.x); o[2] = bf16_lo(a.y); o[3] = bf16_hi(a.y);
+}
+__device__ __forceinline__ void gn_st4(float* p, int64_t i, const float* v) {
+    *reinterpret_cast<float4*>(p + i) = make_float4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ void gn_st4(bf16s* p, int64_t i, const float* v) {
+    uint2 a;
+    a.x = pack_bf16x2(v[0], v[1]);
+    a.y = pack_bf16x2(v[2], v[3]);
+    *reinterpret_cast<uint2*>(p + i) = a;
+}
+
+// VEC: 4 consecutive channels per lane and access (part size % 4 == 0, rows
+// and bases aligned to 4 elements).
+template <typename TG, typename TO, bool VEC>
 __global__ __launch_bounds__(256) void gated_rms_norm_kernel(
     const float* __restrict__ o, const float* __restrict__ w, int wlen,
     const TG* __restrict__ gate, int64_t gs, int gate_act, TO* __restrict__ out, int N,
     int groups, float eps) {
     __shared__ float red[16];
+    constexpr int W = VEC ? 4 : 1;
+    constexpr int NS = GN_NR / W;
     const int t = blockIdx.x;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float* src = o + (int64_t)t * N;
     const TG* gr = gate + (int64_t)t * gs;
     TO* dst = out + (int64_t)t * N;
     const int per = N / groups;
-    if (groups == 1) {
-        float ss = 0.0f;
-        for (int i = threadIdx.x; i < N; i += blockDim.x) ss += src[i] * src[i];
-        ss = block_reduce_sum<4>(ss, red);
-        const float r = 1.0f / sqrtf(ss / (float)N + eps);
-        for (int i = threadIdx.x; i < N; i += blockDim.x) {
-            const float g = ldf(gr, i);
-            const float a = gate_act ? g / (1.0f + expf(-g)) : sigmoidf_(g);
-            stf(dst, i, src[i] * r * w[i] * a);
+    // one part: the block's 256 threads stride it; several: a wave per part
+    const int nth = groups == 1 ? 256 : 64;
+    const int me = groups == 1 ? threadIdx.x : lane;
+    const int gi = groups == 1 ? 0 : blockIdx.y * 4 + wave;
+    if (gi >= groups) return;
+    const int base = gi * per;
+    float vals[GN_NR];
+    float ss = 0.0f;
+#pragma unroll
+    for (int j = 0; j < NS; ++j) {
+        const int i = (me + nth * j) * W;
+#pragma unroll
+        for (int e = 0; e < W; ++e) vals[j * W + e] = 0.0f;
+        if (i < per) {
+            if (VEC) gn_ld4(src, base + i, vals + j * W);
+            else vals[j] = src[base + i];
         }
-        return;
+#pragma unroll
+        for (int e = 0; e < W; ++e) ss += vals[j * W + e] * vals[j * W + e];
     }
-    for (int gi = wave; gi < groups; gi += nw) {
-        const float* s = src + gi * per;
-        float ss = 0.0f;
-        for (int i = lane; i < per; i += 64) ss += s[i] * s[i];
-        ss = wave_reduce_sum(ss);
-        const float r = 1.0f / sqrtf(ss / (float)per + eps);
-        for (int i = lane; i < per; i += 64) {
-            const int c = gi * per + i;
-            const float g = ldf(gr, c);
-            const float a = gate_act ? g / (1.0f + expf(-g)) : sigmoidf_(g);
-            stf(dst, c, s[i] * r * w[wlen == N ? c : i] * a);
-        }
+    for (int i = (me + nth * NS) * W; i < per; i += nth * W)
+#pragma unroll
+        for (int e = 0; e < W; ++e) ss += src[base + i + e] * src[base + i + e];
+    ss = groups == 1 ? block_reduce_sum<4>(ss, red) : wave_reduce_sum(ss);
+    const float r = 1.0f / sqrtf(ss / (float)per + eps);
+    auto emit = [&](int i, const float* x) {
+        const int c = base + i;
+        float g[W], y[W];
+        if (VEC) gn_ld4(gr, c, g);
+        else g[0] = ldf(gr, c);
+#pragma unroll
+        for (int e = 0; e < W; ++e)
+            y[e] = x[e] * r * w[(wlen == N ? c : i) + e] * gate_fn(g[e], gate_act);
+        if (VEC) gn_st4(dst, c, y);
+        else stf(dst, c, y[0]);
+    };
+#pragma unroll
+    for (int j = 0; j < NS; ++j) {
+        const int i = (me + nth * j) * W;
+        if (i < per) emit(i, vals + j * W);
+    }
+    for (int i = (me + nth * NS) * W; i < per; i += nth * W) {
+        float x[W];
+#pragma unroll
+        for (int e = 0; e < W; ++e) x[e] = src[base + i + e];
+        emit(i, x);
     }
 }
 
@@ -283,14 +334,23 @@ extern "C" int oa_gated_rms_norm(void* stream, const void* o, const void* w, int
     if (groups < 1 || N % groups != 0 || (wlen != N && wlen != N / groups)) return -100;
     if (gate_dt != out_dt) return -101;
     hipStream_t s = (hipStream_t)stream;
-    if (out_dt == 1)
-        hipLaunchKernelGGL((gated_rms_norm_kernel<float, float>), dim3(T), dim3(256), 0, s,
-                           (const float*)o, (const float*)w, wlen, (const float*)gate, gs, gate_act,
-                           (float*)out, N, groups, eps);
-    else
-        hipLaunchKernelGGL((gated_rms_norm_kernel<bf16s, bf16s>), dim3(T), dim3(256), 0, s,
-                           (const float*)o, (const float*)w, wlen, (const bf16s*)gate, gs, gate_act,
-                           (bf16s*)out, N, groups, eps);
+    dim3 grid(T, groups == 1 ? 1 : CEIL_DIV(groups, 4));
+    const int esz = out_dt == 1 ? 4 : 2;
+    const bool vec = (N / groups) % 4 == 0 && (uintptr_t)o % 16 == 0 && (uintptr_t)w % 16 == 0 &&
+                     (uintptr_t)gate % (4 * esz) == 0 && gs % 4 == 0 &&
+                     (uintptr_t)out % (4 * esz) == 0;
+#define GN_LAUNCH(TG, V)                                                                       \
+    hipLaunchKernelGGL((gated_rms_norm_kernel<TG, TG, V>), grid, dim3(256), 0, s,               \
+                       (const float*)o, (const float*)w, wlen, (const TG*)gate, gs, gate_act,   \
+                       (TG*)out, N, groups, eps)
+    if (out_dt == 1) {
+        if (vec) GN_LAUNCH(float, true);
+        else GN_LAUNCH(float, false);
+    } else {
+        if (vec) GN_LAUNCH(bf16s, true);
+        else GN_LAUNCH(bf16s, false);
+    }
+#undef GN_LAUNCH
     HIP_CHECK_LAUNCH();
     return 0;
 }

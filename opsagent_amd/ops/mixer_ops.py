@@ -13,6 +13,7 @@ from __future__ import annotations
 
 import ctypes
 import dataclasses
+import os
 from typing import List, Optional, Tuple
 
 import torch
@@ -237,11 +238,13 @@ def attention_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     if (sb.max_chunk == 1 and H // G >= 16 and dt == 0 and D % 16 == 0 and Dv % 16 == 0
             and D <= 256 and Dv <= 256 and (D <= 128 or D % 32 == 0) and nkt >= 4):
         blocks = ntiles * G * ((H // G + 63) // 64)
-        if blocks < 256:
+        if blocks < 128:
             # at most 16: a captured step sizes nkt for the longest context
             # the pool allows, and merging many (mostly empty) partials costs
             # more than the splits save
-            nsplit = int(min(nkt // 2, max(1, 512 // blocks), 16))
+            nsplit = int(min(nkt // 2, max(1, 256 // blocks), 16))
+            if os.environ.get("OPSAGENT_ATTN_DECODE_SPLITS"):
+                nsplit = max(1, min(nkt, int(os.environ["OPSAGENT_ATTN_DECODE_SPLITS"])))
     out = torch.empty(T, H * Dv, dtype=q.dtype, device=q.device)
     part_o = part_ml = None
     if nsplit > 1:
