@@ -284,13 +284,18 @@ class LatentAttentionMixer(nn.Module):
             mx.latent_kv_prepare(proj[:, self.n_q : self.n_q + self.n_kv], self.dkv_norm_w,
                                  self.inv_freq, R, rot, self.eps, k_cache, sb)
         q = proj[:, : self.n_q]
+        # the batched GEMMs over heads read and write token-major rows through
+        # strided views: no head-major copies on either side of the attention
         q_un = q.view(T, H, D + rot)[..., :D].transpose(0, 1)  # [H, T, D]
-        q_lat = torch.bmm(q_un, self.uk_w)                    # [H, T, R]
-        qf = mx.latent_q_assemble(q, q_lat, self.inv_freq, H, D, rot, sb)
+        qf = torch.empty(T, H, R + rot, dtype=proj.dtype, device=proj.device)
+        torch.bmm(q_un, self.uk_w, out=qf[..., :R].transpose(0, 1))
+        mx.latent_q_assemble(q, None, self.inv_freq, H, D, rot, sb, out=qf)
         ctx = mx.attention_paged(qf, k_cache, v_view, sb, self.scale, sinks=self.sinks,
                                  gate_logits=proj[:, self.n_q + self.n_kv :])
-        val = torch.bmm(ctx.view(T, H, R).transpose(0, 1), self.uv_w.transpose(1, 2))
-        return ops.linear(val.transpose(0, 1).reshape(T, H * Dv), self.o_w)
+        val = torch.empty(T, H * Dv, dtype=proj.dtype, device=proj.device)
+        torch.bmm(ctx.view(T, H, R).transpose(0, 1), self.uv_w.transpose(1, 2),
+                  out=val.view(T, H, Dv).transpose(0, 1))
+        return ops.linear(val, self.o_w)
 
     def load(self, get, put, p: str) -> None:
         parts = [get(p + "q")] + ([get(p + "dkv")] if self.own else []) + [get(p + "g")]

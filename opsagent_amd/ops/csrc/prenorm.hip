@@ -248,7 +248,8 @@ extern "C" int oa_latent_kv_prepare(void* stream, const void* dkv, int64_t ds, c
 // ---------------------------------------------------------------------------
 // Queries of latent attention against the cached rows. q [T, H * (D + rot)]
 // holds per head D unrotated and rot rotated channels; q_lat [H, T, rank] is
-// the unrotated part already taken through the key up-projection. out
+// the unrotated part already taken through the key up-projection (null: the
+// caller's batched GEMM has written it into out already). out
 // [T, H, rank + rot] = q_lat beside the part rotated by position. One wave
 // per (token, head).
 template <typename TC>
@@ -266,7 +267,8 @@ __global__ __launch_bounds__(256) void latent_q_assemble_kernel(
     for (int h = blockIdx.y * 4 + wave; h < H; h += gridDim.y * 4) {
         const TC* src = q_lat + ((int64_t)h * T + t) * rank;
         TC* dst = out + ((int64_t)t * H + h) * (rank + rot);
-        for (int i = lane; i < rank; i += 64) dst[i] = src[i];
+        if (q_lat)
+            for (int i = lane; i < rank; i += 64) dst[i] = src[i];
         const TC* qr = q + (int64_t)t * qs + (int64_t)h * (D + rot) + D;
         for (int i = lane; i < npair; i += 64) {
             const float u = ldf(qr, 2 * i), v = ldf(qr, 2 * i + 1);

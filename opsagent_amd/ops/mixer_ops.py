@@ -572,22 +572,36 @@ def latent_kv_prepare(dkv: torch.Tensor, norm_w: torch.Tensor, inv_freq: torch.T
     hip.check(rc, "oa_latent_kv_prepare")
 
 
-def latent_q_assemble(q: torch.Tensor, q_lat: torch.Tensor, inv_freq: torch.Tensor,
-                      H: int, D: int, rot: int, sb: SeqBatch) -> torch.Tensor:
+def latent_q_assemble(q: torch.Tensor, q_lat: Optional[torch.Tensor], inv_freq: torch.Tensor,
+                      H: int, D: int, rot: int, sb: SeqBatch,
+                      out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Queries against the cached latent rows: q [T, H*(D+rot)] (per head D
     unrotated, then rot rotated channels; may be a column slice) and q_lat
     [H, T, rank], the unrotated parts already taken through the key
     up-projection. Returns [T, H, rank + rot]: q_lat beside the part rotated
-    by position (float32 angles)."""
+    by position (float32 angles). With `out` given and q_lat None the latent
+    part is already in out[..., :rank] (a batched GEMM can write it there
+    directly) and only the rotated part is filled in."""
     T = q.shape[0]
-    rank = q_lat.shape[2]
-    assert q_lat.shape[:2] == (H, T) and q_lat.is_contiguous() and q_lat.dtype == q.dtype
+    assert (q_lat is None) == (out is not None)
+    if out is not None:
+        rank = out.shape[2] - rot
+        assert out.shape[:2] == (T, H) and out.is_contiguous() and out.dtype == q.dtype
+    else:
+        rank = q_lat.shape[2]
+        assert q_lat.shape[:2] == (H, T) and q_lat.is_contiguous() and q_lat.dtype == q.dtype
     if not q.is_cuda:
+        if out is not None:
+            out[..., rank:] = torch_ref.latent_q_assemble(
+                q, out[..., :rank].transpose(0, 1), inv_freq, H, D, rot, _positions(sb))[..., rank:]
+            return out
         return torch_ref.latent_q_assemble(q, q_lat, inv_freq, H, D, rot, _positions(sb))
     lib, hip = _lib()
-    out = torch.empty(T, H, rank + rot, dtype=q.dtype, device=q.device)
+    if out is None:
+        out = torch.empty(T, H, rank + rot, dtype=q.dtype, device=q.device)
     rc = lib.oa_latent_q_assemble(
-        hip.current_stream_ptr(), q.data_ptr(), _rows(q), q_lat.data_ptr(),
+        hip.current_stream_ptr(), q.data_ptr(), _rows(q),
+        q_lat.data_ptr() if q_lat is not None else None,
         inv_freq.data_ptr(), inv_freq.numel(), out.data_ptr(), sb.seq_of_t.data_ptr(),
         sb.cu_t.data_ptr(), sb.past_t.data_ptr(), sb.num_seqs, T, H, D, rot, rank, _dt(q))
     hip.check(rc, "oa_latent_q_assemble")

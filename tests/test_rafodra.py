@@ -186,6 +186,11 @@ def test_latent_cache_rows_and_queries(mode, geom):
     for h in range(H):
         assert torch.equal(got[:, h, :R].cpu(), q_lat[h].cpu())
         close(got[:, h, R:], O.rotate_pairs(qq[:, h, D:], pos, rdims, base), dtype, f"query head {h}")
+    # the latent part already in place (written by a batched GEMM): only the rotation is added
+    buf = torch.zeros(T, H, R + rot, dtype=dt, device=dev)
+    buf[..., :R] = q_lat.transpose(0, 1)
+    assert mx.latent_q_assemble(q, None, inv, H, D, rot, sb, out=buf) is buf
+    assert torch.equal(buf, got)
 
 
 def _single_layer(pattern, dtype, seed=0, cfg_fn=make_cfg, **kw):
