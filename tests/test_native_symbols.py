@@ -22,7 +22,7 @@ ENTRY_POINTS = [
     "oa_gemv_fp8_ex", "oa_gemv_fp8_mfma", "oa_gemv_gateup", "oa_gemv_gateup_act",
     "oa_gemv_gateup_ex", "oa_gemv_gateup_fp8", "oa_gemv_rw4", "oa_kv_write",
     "oa_masked_argmax", "oa_masked_argmax_f32", "oa_moe_down", "oa_moe_down_emaj", "oa_moe_gateup",
-    "oa_moe_gateup_emaj", "oa_quant_fp8", "oa_rmsnorm", "oa_rope",
+    "oa_moe_gateup_emaj", "oa_moe_gateup_act", "oa_moe_gateup_emaj_act", "oa_quant_fp8", "oa_rmsnorm", "oa_rope",
     "oa_rope_kv", "oa_silu_mul",
 ]
 
@@ -59,5 +59,7 @@ def test_mixers_library_exports():
               "oa_attn_bias_geometry", "oa_attn_bias_paged", "oa_delta_rule_fused",
               "oa_softcap", "oa_silu_mul_rows", "oa_embed_rows", "oa_dyt_norm",
               "oa_attn_rope_prepare", "oa_act_mul_rows", "oa_route_topk",
-              "oa_moe_pairs_gateup", "oa_moe_pairs_down"]:
+              "oa_moe_pairs_gateup", "oa_moe_pairs_down", "oa_add_layer_norm",
+              "oa_latent_kv_prepare", "oa_latent_q_assemble", "oa_decay_scan",
+              "oa_gated_rms_norm"]:
         assert hasattr(lib, s), f"missing {s}"
