@@ -202,7 +202,10 @@ class MixerSpec:
     sliding window and an optional sink term) | "latent_attention" (softmax
     attention over a cached low-rank latent and one rotated key part shared
     by the heads) | "lightning" (linear attention with one fixed decay per
-    head) | "gla" (linear attention with a learned decay per key channel)."""
+    head) | "gla" (linear attention with a learned decay per key channel) |
+    "diff_attention" (rotary softmax attention in two maps per head over the
+    same values, combined as a difference) | "retention" (rotary linear
+    attention with one fixed decay per head)."""
 
     kind: str
     heads: int
@@ -234,15 +237,29 @@ class MixerSpec:
     # the learned per-channel decay sigmoid(z)^(1/tau) ("gla")
     decay: Optional[List[float]] = None
     tau: float = 1.0
+    # which channels a rotation pairs: "interleaved" (2i, 2i+1) or "half"
+    # (i, i + rot_dims/2); the pairs' order does not change a dot product, so
+    # a checkpoint in the "half" layout has its rows permuted once at load
+    rot_layout: str = "interleaved"
+    # score <- softcap * tanh(score / softcap) before the softmax (None = off)
+    softcap: Optional[float] = None
+    # differential attention: the constant of lambda and of the output scale
+    diff: Optional[float] = None
+    # latent attention: size of the normed latent the queries are projected
+    # through (0 = queries come straight from the input)
+    q_rank: int = 0
+    # output gate read from the mixer input: "head" (one logit per head),
+    # "channel" (one per output channel), "none"
+    gate: str = "head"
 
     @property
     def has_kv(self) -> bool:
-        return self.kind in ("attention", "rotary_window") or (
+        return self.kind in ("attention", "rotary_window", "diff_attention") or (
             self.kind == "latent_attention" and self.kv_from is None)
 
     @property
     def has_state(self) -> bool:
-        return self.kind in ("channel_delta", "lightning", "gla")
+        return self.kind in ("channel_delta", "lightning", "gla", "retention")
 
 
 @dataclasses.dataclass
@@ -258,7 +275,9 @@ class RouterSpec:
     g = min(gate, limit), u = clamp(up, -limit, limit),
     y = g sigmoid(alpha g) (u + 1)); the shared expert has its own limit and,
     with shared_gate, is scaled per token by the sigmoid of a learned
-    projection."""
+    projection. gated=False: an expert is down(act(up x)) with no gate
+    branch (act "relu2": the square of relu). bias: the router adds a learned
+    vector to its logits (it enters scores and choice alike)."""
 
     experts: int
     top: int
@@ -276,6 +295,8 @@ class RouterSpec:
     alpha: float = 1.702
     shared_limit: float = 0.0
     shared_gate: bool = False
+    gated: bool = True
+    bias: bool = False
 
 
 @dataclasses.dataclass
@@ -303,8 +324,21 @@ class HybridSpec:
     # "post_canon": grouped RMS norm on sublayer outputs, sublayers read
     # x + canon(x). "sandwich": a dynamic-tanh norm before and after every
     # sublayer. "pre_norm": a weighted layer norm before every sublayer.
+    # "hyper": pre-norm sublayers (layer norm with weight and bias) around
+    # `streams` residual streams joined by learned hyper-connections.
     layer_style: str = "post_canon"
     embed_scale: float = 1.0
+    streams: int = 1
+    # learned read/mix/write coefficients between the streams (False: the
+    # plain residual sum, which is one stream with all coefficients 1)
+    hyper: bool = False
+    # layers [start, stop) run `times` times in a row with the same weights;
+    # every pass keeps its own keys, values and state
+    loop: Optional[tuple] = None
+    # logits = head(norm(x)) * logit_scale; tied_head: the head is the
+    # embedding table itself (without its scale)
+    logit_scale: float = 1.0
+    tied_head: bool = False
     max_seq_len: int = 1 << 20
     weights_path: Optional[str] = None
 
@@ -314,6 +348,15 @@ class HybridSpec:
     @property
     def num_layers(self) -> int:
         return len(self.layers)
+
+    def layer_runs(self) -> List[int]:
+        """The layers in the order they run (a looped layer once per pass)."""
+        n = len(self.layers)
+        if not self.loop:
+            return list(range(n))
+        start, stop, times = self.loop
+        return (list(range(start)) + list(range(start, stop)) * times
+                + list(range(stop, n)))
 
 
 def povazen_spec_from_dict(cfg: dict, name: str = "povazen") -> HybridSpec:
@@ -611,10 +654,160 @@ def rafodra_config_dict(
             "norm": {"eps": eps}, "vocab": vocab, "width": width}
 
 
+def suzulix_spec_from_dict(cfg: dict, name: str = "suzulix") -> HybridSpec:
+    """Parse a Suzulix config.json dict: pre-norm sublayers (layer norm with
+    weight and bias) on `streams` hyper-connected residual streams; mixers
+    latent attention with a query latent, differential rotary attention with
+    a score soft cap, or retention; routed feed-forwards of ungated
+    squared-relu experts with a biased router and a gated shared expert; a
+    run of layers may loop; the head is the embedding table."""
+    layers = []
+    for i, entry in enumerate(cfg["layers"]):
+        kind, m = entry["type"], entry["mixer"]
+        rot = m.get("rot") or {}
+        if kind == "latent_attention":
+            mixer = MixerSpec(
+                kind=kind, heads=int(m["heads"]), kv_heads=1, dim=int(m["dim"]),
+                vdim=int(m["vdim"]), scale=float(m["scale"]) if "scale" in m else None,
+                rot_dims=int(rot.get("dims", m["rot_dim"])),
+                rot_base=float(rot.get("base", 10000.0)), rot_layout="half",
+                kv_rank=int(m["kv_rank"]), rot_dim=int(m["rot_dim"]),
+                q_rank=int(m.get("q_rank", 0)), sink=False, gate="channel",
+            )
+            if mixer.rot_dims % 2 or mixer.rot_dims > mixer.rot_dim:
+                raise ValueError("rot.dims must be even and at most rot_dim")
+        elif kind == "attention":
+            mixer = MixerSpec(
+                kind="diff_attention", heads=int(m["heads"]), kv_heads=int(m["kv_heads"]),
+                dim=int(m["dim"]), vdim=int(m["vdim"]),
+                scale=float(m["scale"]) if "scale" in m else None,
+                rot_dims=int(rot.get("dims", 0)), rot_base=float(rot.get("base", 10000.0)),
+                rot_layout="interleaved",
+                softcap=float(m["softcap"]) if m.get("softcap") else None,
+                diff=float(m["diff"]), gate="channel",
+            )
+            if mixer.heads % mixer.kv_heads:
+                raise ValueError("heads must be a multiple of kv_heads")
+            if mixer.rot_dims % 2 or mixer.rot_dims > mixer.dim:
+                raise ValueError("rot.dims must be even and at most dim")
+        elif kind == "retention":
+            mixer = MixerSpec(
+                kind=kind, heads=int(m["heads"]), kv_heads=int(m["heads"]), dim=int(m["dim"]),
+                vdim=int(m["vdim"]), decay=[float(d) for d in m["decay"]],
+                rot_dims=int(rot.get("dims", 0)), rot_base=float(rot.get("base", 10000.0)),
+                rot_layout="half", gate="channel",
+            )
+            if len(mixer.decay) != mixer.heads:
+                raise ValueError("retention: one decay per head")
+            if mixer.rot_dims % 2 or mixer.rot_dims > mixer.dim:
+                raise ValueError("rot.dims must be even and at most dim")
+        else:
+            raise ValueError(f"unknown Suzulix layer type {kind!r}")
+        mlp = entry.get("mlp")
+        ls = HybridLayerSpec(mixer=mixer)
+        if mlp is not None:
+            mk = mlp.get("kind", "moe")
+            if mk != "moe":
+                raise ValueError(f"unknown Suzulix feed-forward kind {mk!r}")
+            r = mlp["router"]
+            shared = mlp.get("shared") or {}
+            ls.mlp_kind = "moe"
+            ls.router = RouterSpec(
+                experts=int(r["experts"]), top=int(r["top"]), ff=int(mlp["expert"]["ff"]),
+                score="softmax", correction=False, groups=1, keep=1, scale=1.0,
+                shared_ff=int(shared.get("ff", 0)), rating="max", renorm=True, act="relu2",
+                shared_gate=bool(shared), gated=False, bias=True,
+            )
+            if ls.router.top > ls.router.experts:
+                raise ValueError("router.top exceeds router.experts")
+        layers.append(ls)
+    loop = cfg.get("loop")
+    if loop:
+        start, stop, times = int(loop["start"]), int(loop["stop"]), int(loop["times"])
+        if not (0 <= start <= stop <= len(layers)) or times < 1:
+            raise ValueError("loop: need 0 <= start <= stop <= layers and times >= 1")
+        loop = (start, stop, times) if stop > start and times != 1 else None
+    streams = int(cfg.get("streams", 1))
+    if streams < 1:
+        raise ValueError("streams must be at least 1")
+    return HybridSpec(
+        name=name, architecture="Suzulix", vocab_size=int(cfg["vocab"]),
+        hidden_size=int(cfg["width"]), layers=layers, norm_eps=float(cfg["norm"]["eps"]),
+        layer_style="hyper", embed_scale=float((cfg.get("embedding") or {}).get("scale", 1.0)),
+        streams=streams, hyper="streams" in cfg, loop=loop or None,
+        logit_scale=float(cfg.get("logit_scale", 1.0)), tied_head=True,
+    )
+
+
+def suzulix_config_dict(
+    vocab: int, width: int, pattern: str, heads: int = 4, kv_heads: int = 2, dim: int = 16,
+    vdim: int = 16, kv_rank: int = 24, q_rank: int = 24, rot_dim: int = 8,
+    lat_heads: Optional[int] = None, lat_dim: Optional[int] = None,
+    lat_vdim: Optional[int] = None, rot_dims: Optional[int] = None, rot_base: float = 10000.0,
+    scale: Optional[float] = None, softcap: Optional[float] = 50.0, diff: float = 0.5,
+    ret_heads: Optional[int] = None, ret_dim: Optional[int] = None,
+    ret_vdim: Optional[int] = None, ret_rot_dims: Optional[int] = None,
+    decay: Optional[List[float]] = None, experts: int = 8, top: int = 2, expert_ff: int = 32,
+    shared_ff: int = 0, streams: Optional[int] = 2, loop: Optional[tuple] = None,
+    embed_scale: float = 1.0, logit_scale: float = 1.0, eps: float = 1e-5,
+) -> dict:
+    """A Suzulix config.json dict from a layer pattern, two characters per
+    layer: the mixer 'L' (latent attention), 'A' (differential attention) or
+    'R' (retention), then the feed-forward 'm' (routed experts) or '-'
+    (none). loop = (start, stop, times); streams=None leaves the key out (one
+    plain residual stream)."""
+    if len(pattern) % 2:
+        raise ValueError("pattern: two characters per layer")
+    lh, ld, lv = lat_heads or heads, lat_dim or dim, lat_vdim or vdim
+    rh, rd, rv = ret_heads or heads, ret_dim or dim, ret_vdim or vdim
+    if decay is None:
+        decay = [1.0 - 2.0 ** (-(3 + 2 * h)) for h in range(rh)]
+    layers = []
+    for i in range(0, len(pattern), 2):
+        mk, fk = pattern[i], pattern[i + 1]
+        if mk == "L":
+            mixer = {"heads": lh, "dim": ld, "vdim": lv, "kv_rank": kv_rank, "q_rank": q_rank,
+                     "rot_dim": rot_dim, "rot": {"base": rot_base, "dims": rot_dim},
+                     "scale": scale if scale is not None else (ld + rot_dim) ** -0.5}
+            kind = "latent_attention"
+        elif mk == "A":
+            mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "diff": diff,
+                     "rot": {"base": rot_base, "dims": dim if rot_dims is None else rot_dims},
+                     "scale": scale if scale is not None else dim ** -0.5}
+            if softcap:
+                mixer["softcap"] = softcap
+            kind = "attention"
+        elif mk == "R":
+            mixer = {"heads": rh, "dim": rd, "vdim": rv, "decay": list(decay),
+                     "rot": {"base": rot_base,
+                             "dims": rd if ret_rot_dims is None else ret_rot_dims}}
+            kind = "retention"
+        else:
+            raise ValueError(f"unknown mixer letter {mk!r}")
+        if fk == "m":
+            mlp = {"kind": "moe", "expert": {"ff": expert_ff},
+                   "router": {"experts": experts, "top": top}}
+            if shared_ff:
+                mlp["shared"] = {"ff": shared_ff}
+        elif fk == "-":
+            mlp = None
+        else:
+            raise ValueError(f"unknown feed-forward letter {fk!r}")
+        layers.append({"type": kind, "mixer": mixer, "mlp": mlp})
+    cfg = {"architecture": "Suzulix", "embedding": {"scale": embed_scale}, "layers": layers,
+           "logit_scale": logit_scale, "norm": {"eps": eps}, "vocab": vocab, "width": width}
+    if streams is not None:
+        cfg["streams"] = streams
+    if loop is not None:
+        cfg["loop"] = {"start": loop[0], "stop": loop[1], "times": loop[2]}
+    return cfg
+
+
 # config.json "architecture" -> parser
 ARCHITECTURE_PARSERS = {"Povazen": povazen_spec_from_dict,
                         "Vazilorn": vazilorn_spec_from_dict,
-                        "Rafodra": rafodra_spec_from_dict}
+                        "Rafodra": rafodra_spec_from_dict,
+                        "Suzulix": suzulix_spec_from_dict}
 
 # named hybrid configurations (random-weight benchmarking and tests)
 HYBRID_REGISTRY = {
@@ -668,6 +861,18 @@ HYBRID_REGISTRY = {
     "rafodra-4l4k": lambda: rafodra_config_dict(
         vocab=2048, width=4096, pattern="LdGdAdSd", heads=32, dim=128, vdim=128, ff=14336,
         kv_rank=192, rot_dim=64, lin_heads=32, lin_dim=128, lin_vdim=128),
+    # CPU-test size: every mixer once, a looped pair of layers, three streams
+    "suzulix-tiny": lambda: suzulix_config_dict(
+        vocab=512, width=64, pattern="LmAmRmR-Am", heads=4, kv_heads=2, dim=16, vdim=24,
+        kv_rank=24, q_rank=40, rot_dim=8, lat_dim=16, lat_vdim=8, rot_dims=12, ret_heads=2,
+        ret_dim=32, ret_vdim=16, experts=8, top=3, expert_ff=32, shared_ff=48, streams=3,
+        loop=(1, 3, 2), embed_scale=4.0, logit_scale=0.5),
+    # GPU-smoke size
+    "suzulix-micro": lambda: suzulix_config_dict(
+        vocab=2048, width=1024, pattern="LmAmRmRmLm", heads=8, kv_heads=2, dim=64, vdim=128,
+        kv_rank=128, q_rank=256, rot_dim=32, lat_dim=64, lat_vdim=64, ret_heads=8,
+        ret_dim=128, ret_vdim=128, experts=16, top=4, expert_ff=512, shared_ff=512,
+        streams=2, loop=(0, 2, 2), embed_scale=8.0, logit_scale=0.25),
 }
 
 

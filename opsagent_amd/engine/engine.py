@@ -365,10 +365,13 @@ class LLMEngine:
         kv_gb = float(cfg.get("kv_cache_gb", 0) or 0)
         if self.hybrid:
             esz = 4 if self.dtype == torch.float32 else 2
-            per_token = sum(
-                sh[0] * (sh[1] + (0 if len(sh) > 3 else sh[2]))
-                for sh in self.model.kv_layer_shapes() if sh
-            )
+            def row(sh):
+                mode = sh[3] if len(sh) > 3 else None
+                if mode == "prefix":
+                    return sh[0] * sh[1]
+                return sh[0] * sh[1] + (sh[4] if mode == "vheads" else sh[0]) * sh[2]
+
+            per_token = sum(row(sh) for sh in self.model.kv_layer_shapes() if sh)
             block_bytes = max(1, per_token * self.block_size * esz)
         else:
             hk_local = self.spec.num_kv_heads // self.tp

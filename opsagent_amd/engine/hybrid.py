@@ -1,5 +1,5 @@
 """Hybrid decoders: a per-layer choice of token mixer and feed-forward
-around a float32 residual stream, in two layer styles.
+around a float32 residual stream, in four layer styles.
 
 "post_canon" (the Povazen design): softmax attention with a linear distance
 penalty, or a gated delta rule with per-channel decay.
@@ -21,6 +21,17 @@ attention (learned per-channel decay); dense silu or routed clamped-swish
 feed-forwards.
 Layer:  x <- x + mixer(ln1(x));  x <- x + ff(ln2(x)),
 ln a layer norm with a weight and no bias.
+
+"hyper" (the Suzulix design): latent attention whose queries also pass a
+normed latent, differential attention (two rotary softmax maps per head over
+the same values, soft-capped scores, combined as a difference and normed) or
+retention (rotary linear attention with a fixed per-head decay); routed
+ungated squared-relu experts with a biased router and a gated shared expert.
+Layer: the same pre-norm sublayers (layer norm with weight and bias) on S
+residual streams: a sublayer reads u = sum_s in_s x_s and writes
+x_t <- sum_s mix[s, t] x_s + out_t y; the model's output is the streams' sum.
+A run of layers may loop with the same weights; every pass has its own cache
+and state. The head is the embedding table.
 
 The mixers are modules of their own (BiasedAttentionMixer,
 ChannelDeltaMixer, ...) with every constant a constructor argument, built on the
@@ -61,6 +72,27 @@ def distance_slopes(heads: int, base_exp: float = 8.0) -> torch.Tensor:
     """slope_h = 2^(-base_exp * (h+1) / heads), float32 [heads]."""
     h = torch.arange(1, heads + 1, dtype=torch.float64)
     return torch.pow(2.0, -base_exp * h / heads).to(torch.float32)
+
+
+def half_to_interleaved(rows: torch.Tensor, dims: int) -> torch.Tensor:
+    """Reorder the first `dims` rows of a block from the "half" rotation
+    layout (row i pairs with row i + dims/2) to the interleaved one (row 2i
+    pairs with row 2i+1). Applied alike to the query and key projections it
+    leaves every dot product unchanged."""
+    idx = torch.arange(dims).view(2, dims // 2).t().reshape(-1)
+    return torch.cat([rows[idx], rows[dims:]], 0)
+
+
+def _relayout_heads(w: torch.Tensor, heads: int, dim: int, offset: int, dims: int,
+                    layout: str) -> torch.Tensor:
+    """w [heads * dim, K]: within every head, rows offset .. offset + dims go
+    from `layout` to the interleaved rotation layout."""
+    if layout != "half" or dims == 0:
+        return w
+    w = w.reshape(heads, dim, -1)
+    parts = [torch.cat([w[h, :offset], half_to_interleaved(w[h, offset:], dims)], 0)
+             for h in range(heads)]
+    return torch.stack(parts).reshape(heads * dim, -1)
 
 
 class BiasedAttentionMixer(nn.Module):
@@ -241,7 +273,14 @@ class LatentAttentionMixer(nn.Module):
     A layer with kv_from = j projects no latent: it reads layer j's cache
     rows with its own queries, up-projections, sinks and gates.
 
-    Fused projection rows: q | dkv (own latent only) | gate."""
+    Options, each a MixerSpec field: q_rank > 0 sends the queries through a
+    latent of their own, q = W_uq rms_norm(W_dq h) (weighted); sink=False
+    leaves the sink term out; gate "channel" multiplies the concatenated head
+    outputs elementwise by sigmoid(W_g h) ([heads * vdim] logits) instead of
+    one logit per head; rot_layout "half" names the checkpoint's pairing of
+    rotated channels (rows are reordered once at load).
+
+    Fused projection rows: q (or dq) | dkv (own latent only) | gate."""
 
     def __init__(self, hidden: int, m: MixerSpec, eps: float, dtype, gen):
         super().__init__()
@@ -254,15 +293,24 @@ class LatentAttentionMixer(nn.Module):
         H, D, Dv, R, rot = self.H, self.D, self.Dv, self.R, self.rot
         dev = gen.device
         self.n_q = H * (D + rot)
+        self.q_rank = m.q_rank
+        self.n_in = m.q_rank or self.n_q          # leading projection rows: dq or q
         self.n_kv = R + rot if self.own else 0
+        self.gate = m.gate
+        self.layout, self.rot_dims, self.dtype = m.rot_layout, m.rot_dims, dtype
+        n_gate = {"head": H, "channel": H * Dv, "none": 0}[m.gate]
         std = 1.0 / math.sqrt(hidden)
-        self.proj_w = _param(_rand(gen, self.n_q + self.n_kv + H, hidden, std=std, dtype=dtype))
+        self.proj_w = _param(_rand(gen, self.n_in + self.n_kv + n_gate, hidden, std=std,
+                                   dtype=dtype))
+        if m.q_rank:
+            self.dq_norm_w = _param((1.0 + 0.1 * _rand(gen, m.q_rank)).to(dtype))
+            self.uq_w = _param(_rand(gen, self.n_q, m.q_rank, std=m.q_rank ** -0.5, dtype=dtype))
         if self.own:
             self.dkv_norm_w = _param(1.0 + 0.1 * _rand(gen, R))
         # up-projections per head: uk [H, D, R] (W_uk,h as stored), uv [H, Dv, R]
         self.uk_w = _param(_rand(gen, H, D, R, std=1.0 / math.sqrt(R), dtype=dtype))
         self.uv_w = _param(_rand(gen, H, Dv, R, std=1.0 / math.sqrt(R), dtype=dtype))
-        self.sinks = _param(_rand(gen, H))
+        self.sinks = _param(_rand(gen, H)) if m.sink else None
         self.o_w = _param(_rand(gen, hidden, H * Dv, std=1.0 / math.sqrt(H * Dv), dtype=dtype))
         self.register_buffer("inv_freq", mx.rotary_inv_freq(m.rot_dims, m.rot_base).to(dev),
                              persistent=False)
@@ -279,11 +327,17 @@ class LatentAttentionMixer(nn.Module):
         k_cache, v_view = kv
         T = h.shape[0]
         H, D, Dv, R, rot = self.H, self.D, self.Dv, self.R, self.rot
-        proj = ops.linear(h, self.proj_w)                     # [T, q | dkv | gate]
+        proj = ops.linear(h, self.proj_w)                     # [T, q or dq | dkv | gate]
+        n_in = self.n_in
         if self.own:
-            mx.latent_kv_prepare(proj[:, self.n_q : self.n_q + self.n_kv], self.dkv_norm_w,
+            mx.latent_kv_prepare(proj[:, n_in : n_in + self.n_kv], self.dkv_norm_w,
                                  self.inv_freq, R, rot, self.eps, k_cache, sb)
-        q = proj[:, : self.n_q]
+        if self.q_rank:
+            _, cq = mx.group_rms_norm(proj[:, :n_in], self.dq_norm_w, 1, self.eps)
+            q = ops.linear(cq, self.uq_w)
+        else:
+            q = proj[:, :n_in]
+        gate = proj[:, n_in + self.n_kv :]
         # the batched GEMMs over heads read and write token-major rows through
         # strided views: no head-major copies on either side of the attention
         q_un = q.view(T, H, D + rot)[..., :D].transpose(0, 1)  # [H, T, D]
@@ -291,14 +345,29 @@ class LatentAttentionMixer(nn.Module):
         torch.bmm(q_un, self.uk_w, out=qf[..., :R].transpose(0, 1))
         mx.latent_q_assemble(q, None, self.inv_freq, H, D, rot, sb, out=qf)
         ctx = mx.attention_paged(qf, k_cache, v_view, sb, self.scale, sinks=self.sinks,
-                                 gate_logits=proj[:, self.n_q + self.n_kv :])
+                                 gate_logits=gate if self.gate == "head" else None)
         val = torch.empty(T, H * Dv, dtype=proj.dtype, device=proj.device)
         torch.bmm(ctx.view(T, H, R).transpose(0, 1), self.uv_w.transpose(1, 2),
                   out=val.view(T, H, Dv).transpose(0, 1))
+        if self.gate == "channel":
+            val = mx.combine_norm_gate(val, H, Dv, self.dtype, gate_logits=gate)
         return ops.linear(val, self.o_w)
 
     def load(self, get, put, p: str) -> None:
-        parts = [get(p + "q")] + ([get(p + "dkv")] if self.own else []) + [get(p + "g")]
+        D, rot = self.D, self.rot
+        relay_q = lambda w: _relayout_heads(w, self.H, D + rot, D, self.rot_dims,  # noqa: E731
+                                            self.layout)
+        if self.q_rank:
+            parts = [get(p + "dq")]
+            put(self.dq_norm_w, [get(p + "dq.norm")])
+            put(self.uq_w, [relay_q(get(p + "uq"))])
+        else:
+            parts = [relay_q(get(p + "q"))]
+        if self.own:
+            parts.append(_relayout_heads(get(p + "dkv"), 1, self.R + rot, self.R,
+                                         self.rot_dims, self.layout))
+        if self.gate != "none":
+            parts.append(get(p + "g"))
         put(self.proj_w, parts)
         if self.own:
             put(self.dkv_norm_w, [get(p + "dkv.norm")])
@@ -306,7 +375,142 @@ class LatentAttentionMixer(nn.Module):
                              .to(self.uk_w.device, self.uk_w.dtype))
         self.uv_w.data.copy_(get(p + "uv").reshape(self.H, self.Dv, self.R)
                              .to(self.uv_w.device, self.uv_w.dtype))
-        put(self.sinks, [get(p + "sink")])
+        if self.sinks is not None:
+            put(self.sinks, [get(p + "sink")])
+        put(self.o_w, [get(p + "o")])
+
+
+class DiffAttentionMixer(nn.Module):
+    """Differential attention: every head has two query/key maps over the
+    same values. q = W_q h (heads x 2 x dim), k = W_k h (kv_heads x 2 x dim),
+    v = W_v h (kv_heads x vdim); both maps are rotated by position on their
+    first rot_dims channels; score = q . k * scale, optionally soft-capped
+    (cap * tanh(score / cap)); each map is a causal softmax attention a_m.
+    With lambda = exp(lq1 . lk1) - exp(lq2 . lk2) + diff (one number for the
+    layer), o = a_1 - lambda a_2, divided per head by its root mean square
+    over vdim (eps inside the root, no weight), times (1 - diff), times
+    sigmoid(W_g h) elementwise.
+
+    The two maps are run as 2 * heads ordinary heads against 2 * kv_heads
+    key heads: projection rows are kept map-major ([map, head, dim]) so that
+    the grouped-query rule head // (heads / kv_heads) pairs map m of a query
+    head with map m of its key head, and the cache holds kv_heads value heads
+    which key head g reads as g mod kv_heads.
+
+    Fused projection rows: q | k | v | gate."""
+
+    def __init__(self, hidden: int, m: MixerSpec, eps: float, dtype, gen):
+        super().__init__()
+        self.H, self.G, self.D, self.Dv = m.heads, m.kv_heads, m.dim, m.vdim
+        self.eps, self.dtype = eps, dtype
+        self.scale = float(m.scale) if m.scale is not None else m.dim ** -0.5
+        self.softcap = m.softcap
+        self.diff = float(m.diff if m.diff is not None else 0.0)
+        self.layout, self.rot_dims = m.rot_layout, m.rot_dims
+        H, G, D, Dv = self.H, self.G, self.D, self.Dv
+        dev = gen.device
+        self.n_q, self.n_k, self.n_v = 2 * H * D, 2 * G * D, G * Dv
+        self.proj_w = _param(_rand(gen, self.n_q + self.n_k + self.n_v + H * Dv, hidden,
+                                   std=1.0 / math.sqrt(hidden), dtype=dtype))
+        # lq1 | lk1 | lq2 | lk2
+        self.lam_w = _param(0.3 * _rand(gen, 4, D))
+        self.o_w = _param(_rand(gen, hidden, H * Dv, std=1.0 / math.sqrt(H * Dv), dtype=dtype))
+        self.register_buffer("inv_freq", mx.rotary_inv_freq(m.rot_dims, m.rot_base).to(dev),
+                             persistent=False)
+        self._lam: Optional[float] = None
+
+    def kv_shape(self):
+        return (2 * self.G, self.D, self.Dv, "vheads", self.G)
+
+    def state_shapes(self) -> Dict[str, tuple]:
+        return {}
+
+    def lam(self) -> float:
+        """lambda, from the float32 parameters (a constant of the layer)."""
+        if self._lam is None:
+            w = self.lam_w.detach().float().cpu()
+            self._lam = float(torch.exp((w[0] * w[1]).sum()) - torch.exp((w[2] * w[3]).sum())
+                              + self.diff)
+        return self._lam
+
+    def forward(self, h, sb: mx.SeqBatch, kv, state) -> torch.Tensor:
+        k_cache, v_cache = kv
+        H, G, D, Dv = self.H, self.G, self.D, self.Dv
+        proj = ops.linear(h, self.proj_w)                     # [T, q | k | v | gate]
+        q = mx.attn_rope_prepare(proj, None, None, self.inv_freq, 2 * H, 2 * G, D, Dv, self.eps,
+                                 k_cache, v_cache, sb, v_heads=G)
+        ctx = mx.attention_paged(q, k_cache, v_cache, sb, self.scale, softcap=self.softcap)
+        n = H * Dv                                            # map 1 | map 2
+        y = mx.combine_norm_gate(ctx[:, :n], H, Dv, self.dtype, a2=ctx[:, n:], lam=self.lam(),
+                                 norm=True, eps=self.eps, post_scale=1.0 - self.diff,
+                                 gate_logits=proj[:, self.n_q + self.n_k + self.n_v :])
+        return ops.linear(y, self.o_w)
+
+    def load(self, get, put, p: str) -> None:
+        def map_major(w, heads):      # [head, map, dim] rows -> [map, head, dim]
+            w = _relayout_heads(w, heads * 2, self.D, 0, self.rot_dims, self.layout)
+            return w.reshape(heads, 2, self.D, -1).transpose(0, 1).reshape(2 * heads * self.D, -1)
+
+        put(self.proj_w, [map_major(get(p + "q"), self.H), map_major(get(p + "k"), self.G),
+                          get(p + "v"), get(p + "g")])
+        put(self.lam_w, [get(p + "lq1").reshape(1, -1), get(p + "lk1").reshape(1, -1),
+                         get(p + "lq2").reshape(1, -1), get(p + "lk2").reshape(1, -1)])
+        self._lam = None
+        put(self.o_w, [get(p + "o")])
+
+
+class RetentionMixer(nn.Module):
+    """Retention: linear attention with one fixed decay per head and no
+    softmax or denominator. q = W_q h, k = W_k h (heads x dim) are rotated by
+    position on their first rot_dims channels, k is scaled by dim^-1/2;
+    per head S <- decay_h S + k v^T, o = S^T q with S float32 per-sequence
+    state. Each head's o is divided by its root mean square (no weight) and
+    the concatenated heads are multiplied by silu(W_g h). Rotation and
+    recurrence run on float32 copies of the projections.
+
+    The scale dim^-1/2 is applied to q instead of k: the read-out is linear
+    in both, only the stored state differs by that factor.
+
+    Fused projection rows: q | k | v | gate."""
+
+    def __init__(self, hidden: int, m: MixerSpec, eps: float, dtype, gen):
+        super().__init__()
+        self.H, self.D, self.Dv = m.heads, m.dim, m.vdim
+        self.eps, self.dtype = eps, dtype
+        self.layout, self.rot_dims = m.rot_layout, m.rot_dims
+        H, D, Dv = self.H, self.D, self.Dv
+        self.proj_w = _param(_rand(gen, 2 * H * D + 2 * H * Dv, hidden,
+                                   std=1.0 / math.sqrt(hidden), dtype=dtype))
+        self.o_w = _param(_rand(gen, hidden, H * Dv, std=1.0 / math.sqrt(H * Dv), dtype=dtype))
+        self.register_buffer(
+            "decay", torch.tensor([float(d) for d in m.decay], dtype=torch.float64)
+            .to(torch.float32).to(gen.device), persistent=False)
+        self.register_buffer("inv_freq",
+                             mx.rotary_inv_freq(m.rot_dims, m.rot_base).to(gen.device),
+                             persistent=False)
+
+    def kv_shape(self):
+        return None
+
+    def state_shapes(self) -> Dict[str, tuple]:
+        return {"S": (self.H, self.Dv, self.D)}      # S transposed: [head, value, key]
+
+    def forward(self, h, sb: mx.SeqBatch, kv, state) -> torch.Tensor:
+        H, D, Dv = self.H, self.D, self.Dv
+        n, nv = H * D, H * Dv
+        proj = ops.linear(h, self.proj_w)
+        qkv = mx.rope_rows(proj[:, : 2 * n + nv], 2 * H, D, self.inv_freq, sb)   # float32
+        o = mx.decay_linear_attention(qkv[:, :n], qkv[:, n : 2 * n], qkv[:, 2 * n :],
+                                      state["S"], sb, H, D, Dv, head_decay=self.decay,
+                                      q_scale=D ** -0.5)
+        y = mx.combine_norm_gate(o, H, Dv, self.dtype, norm=True, eps=self.eps,
+                                 gate_logits=proj[:, 2 * n + nv :], gate_act="silu")
+        return ops.linear(y, self.o_w)
+
+    def load(self, get, put, p: str) -> None:
+        relay = lambda w: _relayout_heads(w, self.H, self.D, 0, self.rot_dims,  # noqa: E731
+                                          self.layout)
+        put(self.proj_w, [relay(get(p + "q")), relay(get(p + "k")), get(p + "v"), get(p + "g")])
         put(self.o_w, [get(p + "o")])
 
 
@@ -405,7 +609,8 @@ class GatedLinearAttentionMixer(nn.Module):
 MIXERS = {"attention": BiasedAttentionMixer, "channel_delta": ChannelDeltaMixer,
           "rotary_window": RotaryWindowAttentionMixer,
           "latent_attention": LatentAttentionMixer, "lightning": LightningMixer,
-          "gla": GatedLinearAttentionMixer}
+          "gla": GatedLinearAttentionMixer, "diff_attention": DiffAttentionMixer,
+          "retention": RetentionMixer}
 
 
 class GatedMLP(nn.Module):
@@ -433,6 +638,24 @@ class GatedMLP(nn.Module):
 
     def load(self, get, put, p: str) -> None:
         put(self.gate_up_w, [get(p + "gate"), get(p + "up")])
+        put(self.down_w, [get(p + "down")])
+
+
+class PlainMLP(nn.Module):
+    """down(act(up x)) without a gate branch; act "relu2" (the square of
+    relu) | "silu" | "gelu_tanh"."""
+
+    def __init__(self, hidden: int, ff: int, dtype, gen, act: str = "relu2"):
+        super().__init__()
+        self.ff, self.act = ff, act
+        self.up_w = _param(_rand(gen, ff, hidden, std=1.0 / math.sqrt(hidden), dtype=dtype))
+        self.down_w = _param(_rand(gen, hidden, ff, std=1.0 / math.sqrt(ff), dtype=dtype))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.linear(mx.act_rows(ops.linear(x, self.up_w), self.act), self.down_w)
+
+    def load(self, get, put, p: str) -> None:
+        put(self.up_w, [get(p + "up")])
         put(self.down_w, [get(p + "down")])
 
 
@@ -592,7 +815,90 @@ class PreNormLayer(nn.Module):
             self.mlp.load(get, put, p + "mlp.")
 
 
-LAYER_STYLES = {"post_canon": HybridLayer, "sandwich": SandwichLayer, "pre_norm": PreNormLayer}
+class HyperLayer(nn.Module):
+    """Pre-norm sublayers on S hyper-connected residual streams. Sublayer q
+    (1: mixer, 2: feed-forward) reads u = sum_s in_q[s] x_s, computes
+    y = sublayer(layer_norm(u)) (weight and bias), and writes every stream
+    from the old ones: x_t <- sum_s mix_q[s, t] x_s + out_q[t] y. The write
+    of one sublayer and the read and norm of the next (also the next
+    layer's) are one launch: forward takes the already-normed mixer input
+    and returns the next layer's. Without learned coefficients (hyper=False)
+    all of them are 1 on a single stream: the plain residual sum."""
+
+    def __init__(self, spec: HybridSpec, ls: HybridLayerSpec, dtype, gen):
+        super().__init__()
+        C, S = spec.hidden_size, spec.streams
+        dev = gen.device
+        self.dtype, self.eps, self.hyper = dtype, spec.norm_eps, spec.hyper
+        self.norm1_w = _param(1.0 + 0.05 * _rand(gen, C))
+        self.norm1_b = _param(0.02 * _rand(gen, C))
+        self.mixer = MIXERS[ls.mixer.kind](C, ls.mixer, spec.norm_eps, dtype, gen)
+        self.mlp = None
+        if ls.mlp_kind == "moe":
+            from opsagent_amd.engine.moe import RoutedExperts
+
+            self.mlp = RoutedExperts(C, ls.router, dtype, gen)
+        elif ls.mlp_kind is not None:
+            raise ValueError(f"hyper layers take routed feed-forwards, not {ls.mlp_kind!r}")
+
+        def coeffs(q):
+            if spec.hyper:
+                rd = _param(1.0 / S + 0.1 * _rand(gen, S))
+                wr = _param(1.0 + 0.1 * _rand(gen, S))
+                mix = _param(torch.eye(S, device=dev) + 0.1 * _rand(gen, S, S))
+            else:
+                rd, wr = _param(torch.ones(S, device=dev)), _param(torch.ones(S, device=dev))
+                mix = _param(torch.eye(S, device=dev))
+            setattr(self, f"hc{q}_in", rd)
+            setattr(self, f"hc{q}_out", wr)
+            setattr(self, f"hc{q}_mix", mix)
+
+        coeffs(1)
+        if self.mlp is not None:
+            self.norm2_w = _param(1.0 + 0.05 * _rand(gen, C))
+            self.norm2_b = _param(0.02 * _rand(gen, C))
+            coeffs(2)
+
+    def state_shapes(self) -> Dict[str, tuple]:
+        return dict(self.mixer.state_shapes())
+
+    def first_read(self):
+        return self.hc1_in, self.norm1_w, self.norm1_b
+
+    def forward(self, xs, h, sb: mx.SeqBatch, kv, state, nxt):
+        """xs: float32 streams [T, S, C] (updated in place); h: the normed
+        read of this layer's mixer. nxt: (read, w, b) of what follows (None
+        after the last layer). Returns the next normed read or None."""
+        rd, w, b = nxt if nxt is not None else (None, None, None)
+        y = self.mixer(h, sb, kv, state)
+        if self.mlp is None:
+            return mx.hyper_norm(xs, rd, w, b, self.eps, self.dtype, y=y, mix=self.hc1_mix,
+                                 write=self.hc1_out)
+        h2 = mx.hyper_norm(xs, self.hc2_in, self.norm2_w, self.norm2_b, self.eps, self.dtype,
+                           y=y, mix=self.hc1_mix, write=self.hc1_out)
+        m, shared, gate = self.mlp.forward_parts(h2, decode=sb.max_chunk == 1)
+        return mx.hyper_norm(xs, rd, w, b, self.eps, self.dtype, y=m, mix=self.hc2_mix,
+                             write=self.hc2_out, y2=shared, y2_gate=gate)
+
+    def load(self, get, put, p: str) -> None:
+        put(self.norm1_w, [get(p + "norm1")])
+        put(self.norm1_b, [get(p + "norm1.b")])
+        self.mixer.load(get, put, p + "mix.")
+        subs = [1]
+        if self.mlp is not None:
+            put(self.norm2_w, [get(p + "norm2")])
+            put(self.norm2_b, [get(p + "norm2.b")])
+            self.mlp.load(get, put, p + "mlp.")
+            subs.append(2)
+        if self.hyper:
+            for q in subs:
+                put(getattr(self, f"hc{q}_in"), [get(f"{p}hc{q}.in")])
+                put(getattr(self, f"hc{q}_out"), [get(f"{p}hc{q}.out")])
+                put(getattr(self, f"hc{q}_mix"), [get(f"{p}hc{q}.mix")])
+
+
+LAYER_STYLES = {"post_canon": HybridLayer, "sandwich": SandwichLayer, "pre_norm": PreNormLayer,
+                "hyper": HyperLayer}
 
 
 class HybridForCausalLM(nn.Module):
@@ -610,11 +916,21 @@ class HybridForCausalLM(nn.Module):
         self.embed = _param(_rand(gen, spec.vocab_size, C, dtype=dtype))
         self.sandwich = spec.layer_style == "sandwich"
         self.pre_norm = spec.layer_style == "pre_norm"
+        self.hyper = spec.layer_style == "hyper"
+        # the order the layers run in (a looped layer once per pass); caches
+        # and state are kept per RUN, weights per layer
+        self.runs = spec.layer_runs()
         self.layers = nn.ModuleList(
             [LAYER_STYLES[spec.layer_style](spec, ls, dtype, gen) for ls in spec.layers]
         )
         if self.sandwich:
             self.final_norm = DyTNorm(C, gen)
+        elif self.hyper:
+            self.final_norm_w = _param(torch.ones(C, device=device))
+            self.final_norm_b = _param(torch.zeros(C, device=device))
+            self.register_buffer("sum_read", torch.ones(spec.streams, device=device),
+                                 persistent=False)
+            self.register_buffer("one_read", torch.ones(1, device=device), persistent=False)
         elif self.pre_norm:
             self.final_norm_w = _param(torch.ones(C, device=device))
         else:
@@ -622,7 +938,11 @@ class HybridForCausalLM(nn.Module):
         # layer i reads the cache of layer kv_source[i] (its own unless its
         # mixer names another layer)
         self.kv_source = [getattr(layer.mixer, "kv_source", None) for layer in self.layers]
-        self.lm_head = _param(_rand(gen, spec.vocab_size, C, std=1.0 / math.sqrt(C), dtype=dtype))
+        if spec.tied_head:
+            self.lm_head = self.embed           # the head IS the embedding table
+        else:
+            self.lm_head = _param(_rand(gen, spec.vocab_size, C, std=1.0 / math.sqrt(C),
+                                        dtype=dtype))
         self.vocab_local = spec.vocab_size
         self.to(device)
         # residual stream after every layer of the last forward (debug aid)
@@ -630,15 +950,27 @@ class HybridForCausalLM(nn.Module):
 
     # -- cache geometry the engine sizes its pools from ---------------------
     def kv_layer_shapes(self):
-        return [layer.mixer.kv_shape() for layer in self.layers]
+        return [self.layers[i].mixer.kv_shape() for i in self.runs]
 
     def state_layer_shapes(self) -> List[Dict[str, tuple]]:
-        return [layer.state_shapes() for layer in self.layers]
+        return [self.layers[i].state_shapes() for i in self.runs]
 
     def forward(self, fb: ForwardBatch, kv_caches, state=None) -> torch.Tensor:
         sb = fb.seq_batch
         assert sb is not None and state is not None, "hybrid models run flat multi-sequence steps"
         x = mx.embed_rows(self.embed, fb.input_ids, self.spec.embed_scale)
+        if self.hyper:
+            S, eps = self.spec.streams, self.spec.norm_eps
+            # every stream starts as the embedding output
+            xs = x.unsqueeze(1).expand(-1, S, -1).contiguous() if S > 1 else x.unsqueeze(1)
+            rd, w, b = self.layers[self.runs[0]].first_read()
+            h = mx.hyper_norm(xs, rd, w, b, eps, self.dtype)
+            for r, i in enumerate(self.runs):
+                nxt = self.layers[self.runs[r + 1]].first_read() if r + 1 < len(self.runs) else None
+                h = self.layers[i](xs, h, sb, kv_caches[r], state[r], nxt)
+                if self.trace_layers is not None:
+                    self.trace_layers.append(xs.sum(1))
+            return xs.sum(1) if S > 1 else xs.squeeze(1)
         if self.sandwich or self.pre_norm:
             n = len(self.layers)
             if self.sandwich:
@@ -664,6 +996,10 @@ class HybridForCausalLM(nn.Module):
         if the design caps them)."""
         if self.sandwich:
             normed = mx.dyt_norm(hidden.contiguous(), self.final_norm.params(), self.dtype)
+        elif self.hyper:
+            normed = mx.hyper_norm(hidden.contiguous().unsqueeze(1), self.one_read,
+                                   self.final_norm_w, self.final_norm_b, self.spec.norm_eps,
+                                   self.dtype)
         elif self.pre_norm:
             normed = mx.add_layer_norm(hidden.contiguous(), self.final_norm_w,
                                        self.spec.norm_eps, self.dtype)
@@ -671,6 +1007,8 @@ class HybridForCausalLM(nn.Module):
             _, normed = mx.group_rms_norm(hidden, self.final_norm_w, self.spec.norm_groups,
                                           self.spec.norm_eps, residual=None)
         logits = ops.linear(normed, self.lm_head)
+        if self.spec.logit_scale != 1.0:
+            return logits.float() * self.spec.logit_scale
         if self.spec.logit_softcap is None:
             return logits.float()
         return mx.softcap(logits, self.spec.logit_softcap)
@@ -698,7 +1036,14 @@ class HybridForCausalLM(nn.Module):
             return tensors[name]
 
         put(self.embed, [get("embed")])
-        put(self.lm_head, [get("head")])
+        if not self.spec.tied_head:
+            put(self.lm_head, [get("head")])
+        if self.hyper:
+            put(self.final_norm_w, [get("final.norm")])
+            put(self.final_norm_b, [get("final.norm.b")])
+            for i, layer in enumerate(self.layers):
+                layer.load(get, put, f"l{i}.")
+            return n
         if self.sandwich or self.pre_norm:
             if self.sandwich:
                 self.final_norm.load(get, put, "final.norm")

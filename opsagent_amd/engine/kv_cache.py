@@ -44,7 +44,9 @@ class PagedKVCache:
         recurrent mixer, or a layer that reads another layer's cache); a
         fourth element "prefix" says that the values ARE the first `value
         dim` channels of the keys (one key head): the value tensor is then a
-        view of the key rows and takes no memory. Without layer_shapes every
+        view of the key rows and takes no memory; a fourth element "vheads"
+        with a fifth n says that there are n value heads (n divides kv_heads:
+        key head g reads value head g mod n). Without layer_shapes every
         layer is [kv_heads, head_dim] for both. prefix_caching=False turns block publishing and reuse off: a
         model that also carries recurrent state cannot restart from cached
         keys alone."""
@@ -65,6 +67,10 @@ class PagedKVCache:
             if len(shape) > 3 and shape[3] == "prefix":
                 assert hk == 1 and vdim <= kdim
                 v = k[..., :vdim]
+            elif len(shape) > 4 and shape[3] == "vheads":
+                assert hk % shape[4] == 0
+                v = torch.zeros(num_blocks, block_size, shape[4], vdim, dtype=dtype,
+                                device=device)
             else:
                 v = torch.zeros(num_blocks, block_size, hk, vdim, dtype=dtype, device=device)
             self.layers.append((k, v))

@@ -185,10 +185,11 @@ class RoutedExperts(nn.Module):
     gate activation with its constants, an optional always-on shared expert
     with an optional per-token sigmoid gate whose projection is one more row
     of the float32 router matrix. Router logits, scores and weights are
-    float32.
+    float32. With r.bias the router adds a learned vector to its logits;
+    with r.gated False an expert (and the shared one) is down(act(up x)).
 
-    Expert weights are stacked: w13 [E, 2I, C] (gate rows, then up rows) and
-    w2 [E, C, I]. Few (token, expert) pairs run through two static-shaped
+    Expert weights are stacked: w13 [E, 2I, C] (gate rows, then up rows; up
+    rows alone, [E, I, C], for ungated experts) and w2 [E, C, I]. Few (token, expert) pairs run through two static-shaped
     launches without host sync (hipGraph-capturable); prompt-sized batches
     are sorted by expert and run one library GEMM pair per used expert.
     """
@@ -198,7 +199,7 @@ class RoutedExperts(nn.Module):
         super().__init__()
         if get_tp_size() != 1:
             raise NotImplementedError("routed experts run at tensor-parallel size 1")
-        from opsagent_amd.engine.hybrid import GatedMLP, _param, _rand
+        from opsagent_amd.engine.hybrid import GatedMLP, PlainMLP, _param, _rand
 
         act = act or r.act
         shared_act = act
@@ -211,10 +212,18 @@ class RoutedExperts(nn.Module):
         # router rows, then (optionally) the shared expert's gate row
         self.router_w = _param(_rand(gen, E + int(self.shared_gate), hidden, std=hidden ** -0.5))
         self.correction = _param(0.1 * _rand(gen, E)) if r.correction else None
-        self.w13 = _param(_rand(gen, E, 2 * I, hidden, std=hidden ** -0.5, dtype=dtype))
+        # the shared expert's gate row carries no bias
+        self.router_b = (_param(torch.cat([0.5 * _rand(gen, E),
+                                           torch.zeros(int(self.shared_gate), device=gen.device)]))
+                         if r.bias else None)
+        self.gated = bool(r.gated)
+        self.w13 = _param(_rand(gen, E, (2 if self.gated else 1) * I, hidden,
+                                std=hidden ** -0.5, dtype=dtype))
         self.w2 = _param(_rand(gen, E, hidden, I, std=I ** -0.5, dtype=dtype))
-        self.shared = (GatedMLP(hidden, r.shared_ff, dtype, gen, act=shared_act)
-                       if r.shared_ff else None)
+        self.shared = None
+        if r.shared_ff:
+            self.shared = (GatedMLP(hidden, r.shared_ff, dtype, gen, act=shared_act)
+                           if self.gated else PlainMLP(hidden, r.shared_ff, dtype, gen, act=act))
         # weight bytes one launch pair may stream through the pair kernels
         self.pair_budget = 64 << 20
         self.force_path = None     # "pairs" | "sorted" (tests)
@@ -222,7 +231,7 @@ class RoutedExperts(nn.Module):
     def route(self, x: torch.Tensor, with_gate: bool = False):
         from opsagent_amd.ops import mixer_ops as mx
 
-        logits = F.linear(x.float(), self.router_w)
+        logits = F.linear(x.float(), self.router_w, self.router_b)
         E = self.r.experts
         idx, wts = mx.route_topk(logits[:, :E], self.correction, self.r.top, self.r.groups,
                                  self.r.keep, self.r.scale, self.r.score, self.r.rating,
@@ -250,7 +259,7 @@ class RoutedExperts(nn.Module):
         idx, wts, gate = self.route(x, with_gate=True)
         P, I = T * self.r.top, self.r.ff
         esz = 4 if x.dtype == torch.float32 else 2
-        pairs = (P <= 64 or P * 3 * I * C * esz <= self.pair_budget
+        pairs = (P <= 64 or P * (3 if self.gated else 2) * I * C * esz <= self.pair_budget
                  or (decode and P <= 2048))
         if self.force_path is not None:
             pairs = self.force_path == "pairs"
@@ -265,6 +274,8 @@ class RoutedExperts(nn.Module):
 
         T, C = x.shape
         I, top = self.r.ff, self.r.top
+        if not self.gated:
+            return mx.moe_pairs_plain(x.contiguous(), self.w13, self.w2, idx, wts, self.act)
         fast_act = self.act == "silu" or (isinstance(self.act, tuple)
                                           and self.act[0] == "clamp_swish")
         if (x.is_cuda and x.dtype == torch.bfloat16 and fast_act
@@ -296,7 +307,7 @@ class RoutedExperts(nn.Module):
             if c == 0:
                 continue
             gu = ops.linear(xs[start : start + c], self.w13[e])
-            a = mx.act_mul_rows(gu, I, self.act)
+            a = mx.act_mul_rows(gu, I, self.act) if self.gated else mx.act_rows(gu, self.act)
             ys[start : start + c] = ops.linear(a, self.w2[e]).float()
             start += c
         ys *= w_sorted.unsqueeze(1)
@@ -312,8 +323,14 @@ class RoutedExperts(nn.Module):
             + ([get(p + "shared.sg")] if self.shared_gate else []))
         if self.correction is not None:
             put(self.correction, [get(p + "correction")])
-        w13 = torch.stack([torch.cat([get(f"{p}e{k}.gate"), get(f"{p}e{k}.up")], 0)
-                           for k in range(E)])
+        if self.router_b is not None:
+            put(self.router_b, [get(p + "router.b")]
+                + ([torch.zeros(1)] if self.shared_gate else []))
+        if self.gated:
+            w13 = torch.stack([torch.cat([get(f"{p}e{k}.gate"), get(f"{p}e{k}.up")], 0)
+                               for k in range(E)])
+        else:
+            w13 = torch.stack([get(f"{p}e{k}.up") for k in range(E)])
         w2 = torch.stack([get(f"{p}e{k}.down") for k in range(E)])
         self.w13.data.copy_(w13.to(self.w13.device, self.w13.dtype))
         self.w2.data.copy_(w2.to(self.w2.device, self.w2.dtype))

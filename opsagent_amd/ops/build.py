@@ -29,7 +29,7 @@ SOURCES = [
 
 # the sequence-mixer kernels of hybrid decoders live in a library of their
 # own: a checkout that serves only such a model compiles just what it loads
-MIXER_SOURCES = ["mixers.hip", "blocks.hip", "prenorm.hip", "recurrent.hip"]
+MIXER_SOURCES = ["mixers.hip", "blocks.hip", "prenorm.hip", "recurrent.hip", "hyper.hip"]
 MIXER_OUT = os.path.join(
     os.path.dirname(os.path.abspath(__file__)), "libopsagent_mixers.so"
 )

@@ -106,9 +106,9 @@ extern "C" int oa_dyt_norm(void* stream, const void* y, int64_t ys, int y_dt, co
 // the heads, then the channel pairs (2i, 2i+1), i < nfreq, are rotated by the
 // angle th = position * inv_freq[i], as a plane rotation
 //   [x0'; x1'] = [cos th, -sin th; sin th, cos th] [x0; x1];
-// channels from 2*nfreq on pass unrotated. q goes to q_out [T, H, D], k and
-// the unchanged v (value heads are the last G "heads" of the loop) to their
-// cache slot. The position of token t of sequence b is past[b] + t - cu[b].
+// channels from 2*nfreq on pass unrotated (qw and kw null: no norm, rotation
+// only). q goes to q_out [T, H, D], k and the unchanged v (Gv value heads of
+// Dv channels after the G key heads) to their cache slot. The position of token t of sequence b is past[b] + t - cu[b].
 // Everything between load and store is float32. A lane keeps its pairs in
 // registers (RP_NP pairs: D <= 128 * RP_NP), so every element is read once;
 // the token's cos/sin table is computed once per block into LDS.
@@ -137,7 +137,7 @@ __global__ __launch_bounds__(256) void attn_rope_prepare_kernel(
     const float* __restrict__ kw, const float* __restrict__ inv_freq, int nfreq,
     TC* __restrict__ q_out, TC* __restrict__ k_cache, TC* __restrict__ v_cache,
     const int* __restrict__ slot_mapping, const int* __restrict__ seq_of,
-    const int* __restrict__ cu, const int* __restrict__ past, int B, int H, int G, int D,
+    const int* __restrict__ cu, const int* __restrict__ past, int B, int H, int G, int Gv, int D,
     int Dv, float eps) {
     const int t = blockIdx.x;
     if (t >= cu[B]) return;  // padding row of a fixed-size (captured) launch
@@ -189,7 +189,7 @@ __global__ __launch_bounds__(256) void attn_rope_prepare_kernel(
 #pragma unroll
             for (int j = 0; j < RP_NP; ++j) ss += u[k][j] * u[k][j] + v[k][j] * v[k][j];
             ss = wave_reduce_sum(ss);
-            const float rn = 1.0f / sqrtf(ss / (float)D + eps);
+            const float rn = qw ? 1.0f / sqrtf(ss / (float)D + eps) : 1.0f;
             const bool is_q = hd < H;
             TC* dst = is_q ? q_out + ((int64_t)t * H + hd) * D
                            : k_cache + (slot * G + (hd - H)) * D;
@@ -198,8 +198,8 @@ __global__ __launch_bounds__(256) void attn_rope_prepare_kernel(
                 const int i = lane + 64 * j;
                 if (i >= npair) continue;
                 const float* w = is_q ? qw : kw;
-                const float a = u[k][j] * rn * w[2 * i];
-                const float c = (2 * i + 1 < D) ? v[k][j] * rn * w[2 * i + 1] : 0.0f;
+                const float a = w ? u[k][j] * rn * w[2 * i] : u[k][j];
+                const float c = (2 * i + 1 < D) ? (w ? v[k][j] * rn * w[2 * i + 1] : v[k][j]) : 0.0f;
                 const float ra = a * cs[i] - c * sn[i];
                 const float rc = c * cs[i] + a * sn[i];
                 if (PAIRED) {
@@ -211,10 +211,10 @@ __global__ __launch_bounds__(256) void attn_rope_prepare_kernel(
             }
         }
     }
-    // values: a plain copy of G*Dv contiguous columns to the token's slot
+    // values: a plain copy of Gv*Dv contiguous columns to the token's slot
     const TC* vsrc = row + (int64_t)nh * D;
-    TC* vdst = v_cache + slot * (int64_t)(G * Dv);
-    const int nv = G * Dv, tid = blockIdx.y * blockDim.x + threadIdx.x, nt = gridDim.y * blockDim.x;
+    TC* vdst = v_cache + slot * (int64_t)(Gv * Dv);
+    const int nv = Gv * Dv, tid = blockIdx.y * blockDim.x + threadIdx.x, nt = gridDim.y * blockDim.x;
     if (PAIRED) {
         for (int i = tid; 2 * i < nv; i += nt) {
             float a, c;
@@ -239,7 +239,7 @@ __global__ __launch_bounds__(256) void attn_rope_prepare_vec_kernel(
     const float* __restrict__ kw, const float* __restrict__ inv_freq, int nfreq,
     TC* __restrict__ q_out, TC* __restrict__ k_cache, TC* __restrict__ v_cache,
     const int* __restrict__ slot_mapping, const int* __restrict__ seq_of,
-    const int* __restrict__ cu, const int* __restrict__ past, int B, int H, int G, int D,
+    const int* __restrict__ cu, const int* __restrict__ past, int B, int H, int G, int Gv, int D,
     int Dv, float eps) {
     extern __shared__ float lds[];
     const int npair = D / 2;
@@ -263,8 +263,13 @@ __global__ __launch_bounds__(256) void attn_rope_prepare_vec_kernel(
     const int sub = lane / lph, ch = (lane % lph) * 8;
     const int nh = H + G;
     float wq[8], wk[8];
-    ld8(qw, ch, wq);
-    ld8(kw, ch, wk);
+    if (qw) {
+        ld8(qw, ch, wq);
+        ld8(kw, ch, wk);
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) wq[e] = wk[e] = 1.0f;
+    }
     const int step = gridDim.y * 4 * hpw;
     for (int h0 = (blockIdx.y * 4 + wave) * hpw + sub; h0 < nh + step * RV_IT; h0 += step * RV_IT) {
         if (h0 - sub >= nh) break;                   // uniform over the wave
@@ -286,7 +291,7 @@ __global__ __launch_bounds__(256) void attn_rope_prepare_vec_kernel(
             for (int e = 0; e < 8; ++e) ss += x[k][e] * x[k][e];
             for (int off = lph >> 1; off > 0; off >>= 1) ss += __shfl_xor(ss, off, WAVE);
             if (hd >= nh) continue;
-            const float rn = 1.0f / sqrtf(ss / (float)D + eps);
+            const float rn = qw ? 1.0f / sqrtf(ss / (float)D + eps) : 1.0f;
             const bool is_q = hd < H;
             float o[8];
 #pragma unroll
@@ -302,8 +307,8 @@ __global__ __launch_bounds__(256) void attn_rope_prepare_vec_kernel(
         }
     }
     const TC* vsrc = row + (int64_t)nh * D;
-    TC* vdst = v_cache + slot * (int64_t)(G * Dv);
-    const int nv = G * Dv;
+    TC* vdst = v_cache + slot * (int64_t)(Gv * Dv);
+    const int nv = Gv * Dv;
     for (int i = (blockIdx.y * blockDim.x + threadIdx.x) * 8; i < nv; i += gridDim.y * blockDim.x * 8) {
         float tmp[8];
         ld8(vsrc, i, tmp);
@@ -315,10 +320,12 @@ extern "C" int oa_attn_rope_prepare(void* stream, const void* qkv, int64_t qs, c
                                     const void* kw, const void* inv_freq, int nfreq,
                                     void* q_out, void* k_cache, void* v_cache,
                                     const void* slot_mapping, const void* seq_of, const void* cu,
-                                    const void* past, int B, int T, int H, int G, int D, int Dv,
-                                    float eps, int dt) {
+                                    const void* past, int B, int T, int H, int G, int Gv, int D,
+                                    int Dv, float eps, int dt) {
+    // qw, kw both null: no norm, rotation only. Gv value heads follow the key heads.
     if (T <= 0) return 0;
-    if (2 * nfreq > D || H < 1 || G < 1 || D > 128 * RP_NP) return -100;
+    if (2 * nfreq > D || H < 1 || G < 1 || Gv < 1 || D > 128 * RP_NP || (qw == nullptr) != (kw == nullptr))
+        return -100;
     hipStream_t s = (hipStream_t)stream;
     const int esz = dt == 1 ? 4 : 2;
     const bool paired = D % 2 == 0 && Dv % 2 == 0 && qs % 2 == 0 && (uintptr_t)qkv % (2 * esz) == 0 &&
@@ -331,7 +338,7 @@ extern "C" int oa_attn_rope_prepare(void* stream, const void* qkv, int64_t qs, c
 #define RP_ARGS(TC)                                                                            \
     (const TC*)qkv, qs, (const float*)qw, (const float*)kw, (const float*)inv_freq, nfreq,     \
         (TC*)q_out, (TC*)k_cache, (TC*)v_cache, (const int*)slot_mapping, (const int*)seq_of,  \
-        (const int*)cu, (const int*)past, B, H, G, D, Dv, eps
+        (const int*)cu, (const int*)past, B, H, G, Gv, D, Dv, eps
 #define RP(TC)                                                                                 \
     do {                                                                                       \
         if (paired) hipLaunchKernelGGL((attn_rope_prepare_kernel<TC, true>), dim3(T, ny),      \

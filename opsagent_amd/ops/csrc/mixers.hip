@@ -406,6 +406,8 @@ __global__ __launch_bounds__(256) void attn_prepare_vec_kernel(
 //   window > 0: only keys j > i - window are visible (the last `window`
 //                 positions up to the query); key tiles that end before
 //                 that range are never visited
+//   softcap > 0: q_i . k_j * scale is replaced by softcap * tanh(that / softcap)
+//   Gv value heads (Gv divides G): key head g reads value head g mod Gv
 //   sinks given: Z_i,h = sum_j exp(score(i, j)) + exp(sink_h): the sink
 //                 enlarges the normaliser only, contributes no value
 //                 vector, and `scale` is not applied to it
@@ -430,7 +432,7 @@ __global__ __launch_bounds__(256) void attn_bias_paged_kernel(
     const int* __restrict__ block_table, int max_blocks, int block_size,
     const float* __restrict__ slopes, const float* __restrict__ sinks, int B, int H, int G,
     int D, int Dv, int TQ, int KT, int kstride, float scale, int nsplit, int RB, int window,
-    int64_t vrow) {
+    int64_t vrow, int Gv, float softcap) {
     extern __shared__ float lds[];
     // a block takes up to RB of the H/G query heads of one kv head
     const int hgroups = (H / G + RB - 1) / RB;
@@ -491,7 +493,7 @@ __global__ __launch_bounds__(256) void attn_bias_paged_kernel(
             const int j = i / Dv, d = i % Dv;
             const int key = k0 + j;
             const int64_t slot = (int64_t)bt[key / block_size] * block_size + key % block_size;
-            Vs[j * Dv + d] = v_cache[slot * vrow + g * Dv + d];
+            Vs[j * Dv + d] = v_cache[slot * vrow + (g % Gv) * Dv + d];
         }
         __syncthreads();
 #pragma unroll
@@ -508,6 +510,7 @@ __global__ __launch_bounds__(256) void attn_bias_paged_kernel(
                 const TC* kr = Ks + lane * kstride;
                 float a = 0.0f;
                 for (int d = 0; d < D; ++d) a += qr[d] * ldf(kr, d);
+                if (softcap > 0.0f) a = softcap * tanhf(a / softcap);
                 s = a - slope * (float)(pos - (k0 + lane));
             }
             const float mx = fmaxf(m[ri], wave_reduce_max(s));
@@ -597,7 +600,8 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
     const int* __restrict__ cu, const int* __restrict__ past,
     const int* __restrict__ block_table, int max_blocks, int block_size,
     const float* __restrict__ slopes, const float* __restrict__ sinks, int B, int H, int G,
-    int D, int Dv, int HB, float scale, int nsplit, int window, int vrow, int hrows) {
+    int D, int Dv, int HB, float scale, int nsplit, int window, int vrow, int hrows, int Gv,
+    float softcap) {
     // hrows (decode steps of many query heads per kv head): a step brings one
     // token per sequence, so the 16 columns of a wave's tile are 16 HEADS at
     // that token's position instead of 16 tokens of one head; a block covers
@@ -651,6 +655,10 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
     const float LOG2E = 1.4426950408889634f;
     const float slope = slopes ? slopes[h] * LOG2E : 0.0f;
     const float scale2 = scale * LOG2E;
+    // soft cap: cap * tanh(s / cap) = cap - 2 cap / (exp(2 s / cap) + 1), here
+    // with s = raw * scale and the result in the exp2 domain
+    const float cap_in = softcap > 0.0f ? 2.0f * scale * LOG2E / softcap : 0.0f;
+    const float cap_out = softcap * LOG2E;
     // window as a bound that no position reaches when there is none
     const int wlim = window > 0 ? window : 0x7fffffff;
 
@@ -711,7 +719,7 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
         const int64_t sk_ = okk ? ((int64_t)bt[keyk >> bsh] << bsh) + (keyk & bmask) : 0;
         const int64_t sv_ = okv ? ((int64_t)bt[keyv >> bsh] << bsh) + (keyv & bmask) : 0;
         const bf16s* kp = k_cache + (sk_ * G + g) * D;
-        const bf16s* vp = v_cache + (sv_ * vrow + g * Dv);
+        const bf16s* vp = v_cache + (sv_ * vrow + (g % Gv) * Dv);
 #pragma unroll
         for (int u = 0; u < KC; ++u) {
             const int c = kc0 + 4 * u;
@@ -797,7 +805,14 @@ __global__ __launch_bounds__(256) void attn_bias_mfma_kernel(
             for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
-                    float v = fmaf(sc[u][mt][r], scale2, kbias[mt][r] - base);
+                    float v;
+                    if (softcap > 0.0f) {
+                        const float e2 = __builtin_amdgcn_exp2f(sc[u][mt][r] * cap_in);
+                        v = cap_out - 2.0f * cap_out * __builtin_amdgcn_rcpf(e2 + 1.0f)
+                            + (kbias[mt][r] - base);
+                    } else {
+                        v = fmaf(sc[u][mt][r], scale2, kbias[mt][r] - base);
+                    }
                     if (diag) {
                         const int key = k0 + 16 * mt + 4 * lg + r;
                         v = (key <= pos[u] && key > pos[u] - wlim) ? v : -INFINITY;
@@ -1416,7 +1431,7 @@ static void launch_attn_mfma(hipStream_t s, dim3 grid, int lds_bytes, const void
                              const void* block_table, int max_blocks, int block_size,
                              const void* slopes, const void* sinks, int B, int H, int G, int D,
                              int Dv, int HB, float scale, int nsplit, int window, int64_t vrow,
-                             int hrows) {
+                             int hrows, int Gv, float softcap) {
     if (lds_bytes > 48 * 1024)
         (void)hipFuncSetAttribute((const void*)attn_bias_mfma_kernel<MAXD, MAXDV, QK32, NT>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes);
@@ -1425,7 +1440,7 @@ static void launch_attn_mfma(hipStream_t s, dim3 grid, int lds_bytes, const void
                        (const bf16s*)v_cache, (bf16s*)out, (float*)part_o, (float*)part_ml,
                        (const int*)cu, (const int*)past, (const int*)block_table, max_blocks,
                        block_size, (const float*)slopes, (const float*)sinks, B, H, G, D, Dv, HB,
-                       scale, nsplit, window, (int)vrow, hrows);
+                       scale, nsplit, window, (int)vrow, hrows, Gv, softcap);
 }
 
 // ntiles = sum_b ceil(n_b / TQ) (host-computed). part_* may be null when nsplit == 1.
@@ -1435,13 +1450,14 @@ extern "C" int oa_attn_bias_paged(void* stream, const void* q, const void* gate,
                                   const void* block_table, int max_blocks, int block_size,
                                   const void* slopes, const void* sinks, int T, int B, int ntiles,
                                   int H, int G, int D, int Dv, float scale, int nsplit, int dt,
-                                  int max_chunk, int window, int64_t vrow) {
+                                  int max_chunk, int window, int64_t vrow, int Gv, float softcap) {
     // vrow: elements between the value rows of consecutive cache slots
-    // (G * Dv for a cache of its own; more when the values are the leading
-    // channels of wider rows)
+    // (Gv * Dv for a cache of its own; more when the values are the leading
+    // channels of wider rows). Gv value heads: key head g reads value head
+    // g mod Gv. softcap > 0: score <- softcap * tanh(score / softcap).
     if (T <= 0 || ntiles <= 0) return 0;
     if (window < 0) return -105;
-    if (vrow < (int64_t)G * Dv) return -106;
+    if (Gv < 1 || G % Gv != 0 || vrow < (int64_t)Gv * Dv) return -106;
     int TQ, KT, ks, lds_bytes;
     int rc = oa_attn_bias_geometry(H, G, D, Dv, dt, max_chunk, &TQ, &KT, &ks, &lds_bytes);
     if (rc) return rc;
@@ -1456,7 +1472,8 @@ extern "C" int oa_attn_bias_paged(void* stream, const void* q, const void* gate,
         dim3 grid(ntiles, hrows ? G * CEIL_DIV(R, 64) : G * (R / HB), nsplit);
 #define MF_ARGS                                                                                   \
     s, grid, lds_bytes, q, gate, gs, k_cache, v_cache, out, part_o, part_ml, cu, past, block_table, \
-        max_blocks, block_size, slopes, sinks, B, H, G, D, Dv, HB, scale, nsplit, window, vrow, hrows
+        max_blocks, block_size, slopes, sinks, B, H, G, D, Dv, HB, scale, nsplit, window, vrow, hrows, \
+        Gv, softcap
 #define MF(A, Bv)                                                               \
     do {                                                                        \
         if (D % 32 == 0) launch_attn_mfma<A, Bv, true, 1>(MF_ARGS);             \
@@ -1482,7 +1499,8 @@ extern "C" int oa_attn_bias_paged(void* stream, const void* q, const void* gate,
     (const TC*)q, (const TC*)gate, gs, (const TC*)k_cache, (const TC*)v_cache, (TC*)out,  \
         (float*)part_o, (float*)part_ml, (const int*)cu, (const int*)past,                \
         (const int*)block_table, max_blocks, block_size, (const float*)slopes,            \
-        (const float*)sinks, B, H, G, D, Dv, TQ, KT, ks, scale, nsplit, rb, window, vrow
+        (const float*)sinks, B, H, G, D, Dv, TQ, KT, ks, scale, nsplit, rb, window, vrow, Gv,  \
+        softcap
         if (dt == 1)
             hipLaunchKernelGGL((attn_bias_paged_kernel<float>), grid, blk, lds_bytes, s, AT_ARGS(float));
         else

@@ -129,10 +129,10 @@ def _declare_mixers(lib: ctypes.CDLL) -> None:
         "oa_attn_prepare": [p, p, i64, p, p, p, p, p, p, p, p, i, i, i, i, i, i, f, i],
         "oa_attn_bias_geometry": [i, i, i, i, i, i, ip, ip, ip, ip],
         "oa_attn_bias_paged": [p, p, p, i64, p, p, p, p, p, p, p, p, i, i, p, p,
-                               i, i, i, i, i, i, i, f, i, i, i, i, i64],
+                               i, i, i, i, i, i, i, f, i, i, i, i, i64, i, f],
         "oa_dyt_norm": [p, p, i64, i, p, p, p, p, p, p, p, p, i, i, i],
         "oa_attn_rope_prepare": [p, p, i64, p, p, p, i, p, p, p, p, p, p, p, i, i,
-                                 i, i, i, i, f, i],
+                                 i, i, i, i, i, f, i],
         "oa_act_mul_rows": [p, p, p, i64, i, i, i, f, f],
         "oa_route_topk": [p, p, i64, p, p, p, i, i, i, i, i, f, i, i, i],
         "oa_moe_pairs_gateup": [p, p, p, p, p, i, i, i, i, i, i, i, f, f],
@@ -148,6 +148,11 @@ def _declare_mixers(lib: ctypes.CDLL) -> None:
         "oa_softcap": [p, p, p, i64, f, i],
         "oa_silu_mul_rows": [p, p, p, i64, i, i],
         "oa_embed_rows": [p, p, p, p, i, i, i, f],
+        "oa_hyper_norm": [p, p, i, p, i64, i, p, i64, i, p, i64, p, p, p, p, p, p, i, i, i, f],
+        "oa_rope_rows": [p, p, i64, i, p, i, i, i, p, i, p, p, p, i, i],
+        "oa_combine_norm_gate": [p, p, i64, i, p, i64, f, p, i64, i, p, i, i, i, i, i, f, f],
+        "oa_act_rows": [p, p, p, i64, i, i],
+        "oa_moe_pairs_up": [p, p, p, p, p, i, i, i, i, i, i, i],
     }
     for name, args in sigs.items():
         fn = getattr(lib, name)

@@ -203,24 +203,32 @@ def attention_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
                     sb: SeqBatch, scale: float, slopes: Optional[torch.Tensor] = None,
                     gate_logits: Optional[torch.Tensor] = None,
                     window: Optional[int] = None,
-                    sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    sinks: Optional[torch.Tensor] = None,
+                    softcap: Optional[float] = None) -> torch.Tensor:
     """Causal softmax attention over each sequence's cached keys, score
     q.k*scale. Options, each a parameter: `slopes` [H] float32 subtracts
     slope_h*(i-j); `window` hides keys with i - j >= window; `sinks` [H]
     float32 enlarges head h's softmax normaliser by exp(sink_h) and leaves
-    the numerator alone;
+    the numerator alone; `softcap` replaces the scaled score by
+    softcap * tanh(score / softcap);
     `gate_logits` [T,H] (may be a column slice) scales each head's output by
-    its sigmoid. q [T,H,D]. Returns [T, H*Dv]."""
+    its sigmoid. q [T,H,D]. The cache may hold fewer value heads than key
+    heads (Gv divides G): key head g reads value head g mod Gv.
+    Returns [T, H*Dv]."""
     T, H, D = q.shape
-    nb, bs, G, Dv = v_cache.shape
+    nb, bs, Gv, Dv = v_cache.shape
+    G = k_cache.shape[2]
     window = int(window) if window else 0
+    softcap = float(softcap) if softcap else 0.0
+    assert G % Gv == 0 and H % G == 0
     # v_cache may be a view of the leading channels of wider rows (values
     # that are a prefix of the cached keys): its token stride is passed on
-    assert v_cache.stride(3) == 1 and (G == 1 or v_cache.stride(2) == Dv)
+    assert v_cache.stride(3) == 1 and (Gv == 1 or v_cache.stride(2) == Dv)
     assert v_cache.stride(0) == bs * v_cache.stride(1)
     if not q.is_cuda:
         return torch_ref.attention_paged(q, k_cache, v_cache, sb.cu, sb.past, sb.block_table,
-                                         scale, slopes, gate_logits, window or None, sinks)
+                                         scale, slopes, gate_logits, window or None, sinks,
+                                         softcap or None)
     lib, hip = _lib()
     dt = _dt(q)
     TQ, KT = attn_geometry(H, G, D, Dv, dt, sb.max_chunk)
@@ -265,7 +273,7 @@ def attention_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         sb.block_table.shape[1], bs, slopes.data_ptr() if slopes is not None else None,
         sinks.data_ptr() if sinks is not None else None,
         T, sb.num_seqs, ntiles, H, G, D, Dv,
-        float(scale), nsplit, dt, sb.max_chunk, window, v_cache.stride(1))
+        float(scale), nsplit, dt, sb.max_chunk, window, v_cache.stride(1), Gv, softcap)
     hip.check(rc, "oa_attn_bias_paged")
     return out
 
@@ -330,39 +338,44 @@ def rotary_inv_freq(dims: int, base: float, scaling: Optional[dict] = None) -> t
     return torch.tensor(out, dtype=torch.float32)
 
 
-def attn_rope_prepare(qkv: torch.Tensor, q_norm_w: torch.Tensor, k_norm_w: torch.Tensor,
+def attn_rope_prepare(qkv: torch.Tensor, q_norm_w: Optional[torch.Tensor],
+                      k_norm_w: Optional[torch.Tensor],
                       inv_freq: torch.Tensor, H: int, G: int, D: int, Dv: int, eps: float,
-                      k_cache: torch.Tensor, v_cache: torch.Tensor, sb: SeqBatch) -> torch.Tensor:
-    """qkv [T, >= H*D + G*D + G*Dv] (q | k | v columns). RMS norm of every
-    query and key head over its D channels with the float32 weights [D]
-    (shared by heads), then rotation of the channel pairs (2i, 2i+1),
-    i < len(inv_freq), by position * inv_freq[i] — all in float32; k and v
-    are written to their pages; returns q [T, H, D]."""
+                      k_cache: torch.Tensor, v_cache: torch.Tensor, sb: SeqBatch,
+                      v_heads: Optional[int] = None) -> torch.Tensor:
+    """qkv [T, >= H*D + G*D + Gv*Dv] (q | k | v columns; Gv = v_heads or G).
+    RMS norm of every query and key head over its D channels with the float32
+    weights [D] (shared by heads; both None: no norm), then rotation of the
+    channel pairs (2i, 2i+1), i < len(inv_freq), by position * inv_freq[i] —
+    all in float32; k and v are written to their pages; returns q [T, H, D]."""
     T = qkv.shape[0]
-    assert 2 * inv_freq.numel() <= D
+    Gv = v_heads or G
+    assert 2 * inv_freq.numel() <= D and (q_norm_w is None) == (k_norm_w is None)
     if not qkv.is_cuda:
-        pos = torch.tensor([sb.past[b] + i for b in range(sb.num_seqs)
-                            for i in range(sb.cu[b + 1] - sb.cu[b])], dtype=torch.float32)
         return torch_ref.attn_rope_prepare(qkv, q_norm_w, k_norm_w, inv_freq, H, G, D, Dv, eps,
-                                           k_cache, v_cache, pos, sb.slot_mapping)
+                                           k_cache, v_cache, _positions(sb), sb.slot_mapping,
+                                           Gv)
     lib, hip = _lib()
     assert k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype
-    assert k_cache.shape[2:] == (G, D) and v_cache.shape[2:] == (G, Dv)
+    assert k_cache.shape[2:] == (G, D) and v_cache.shape[2:] == (Gv, Dv)
+    assert k_cache.is_contiguous() and v_cache.is_contiguous()
     for t in (q_norm_w, k_norm_w, inv_freq):
-        assert t.dtype == torch.float32 and t.is_contiguous()
-    assert q_norm_w.numel() == D and k_norm_w.numel() == D
+        assert t is None or (t.dtype == torch.float32 and t.is_contiguous())
+    assert q_norm_w is None or (q_norm_w.numel() == D and k_norm_w.numel() == D)
     q = torch.empty(T, H, D, dtype=qkv.dtype, device=qkv.device)
     rc = lib.oa_attn_rope_prepare(
-        hip.current_stream_ptr(), qkv.data_ptr(), _rows(qkv), q_norm_w.data_ptr(),
-        k_norm_w.data_ptr(), inv_freq.data_ptr(), inv_freq.numel(), q.data_ptr(),
+        hip.current_stream_ptr(), qkv.data_ptr(), _rows(qkv),
+        q_norm_w.data_ptr() if q_norm_w is not None else None,
+        k_norm_w.data_ptr() if k_norm_w is not None else None,
+        inv_freq.data_ptr(), inv_freq.numel(), q.data_ptr(),
         k_cache.data_ptr(), v_cache.data_ptr(), sb.slot_mapping.data_ptr(),
         sb.seq_of_t.data_ptr(), sb.cu_t.data_ptr(), sb.past_t.data_ptr(), sb.num_seqs, T,
-        H, G, D, Dv, eps, _dt(qkv))
+        H, G, Gv, D, Dv, eps, _dt(qkv))
     hip.check(rc, "oa_attn_rope_prepare")
     return q
 
 
-ACTS = {"silu": 0, "gelu_tanh": 1, "clamp_swish": 2}
+ACTS = {"silu": 0, "gelu_tanh": 1, "clamp_swish": 2, "relu2": 3}
 
 
 def act_args(act) -> Tuple[int, float, float]:
@@ -710,4 +723,137 @@ def silu_mul_rows(gu: torch.Tensor, inter: int) -> torch.Tensor:
     out = torch.empty(*gu.shape[:-1], inter, dtype=gu.dtype, device=gu.device)
     hip.check(lib.oa_silu_mul_rows(hip.current_stream_ptr(), gu.data_ptr(), out.data_ptr(),
                                    M, inter, _dt(gu)), "oa_silu_mul_rows")
+    return out
+
+
+def hyper_norm(streams: torch.Tensor, read: Optional[torch.Tensor], w: Optional[torch.Tensor],
+               b: Optional[torch.Tensor], eps: float, out_dtype,
+               y: Optional[torch.Tensor] = None, mix: Optional[torch.Tensor] = None,
+               write: Optional[torch.Tensor] = None, y2: Optional[torch.Tensor] = None,
+               y2_gate: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """One launch for a sublayer's write into hyper-connected residual streams
+    and the read and layer norm before the next sublayer. streams float32
+    [T, S, C], in place. With y [T, C] (plus sigmoid(y2_gate) * y2, as in
+    add_layer_norm), mix float32 [S, S] indexed [from, to] and write float32
+    [S]:  new_t = sum_s mix[s, t] old_s + write[t] * y, every stream from the
+    old ones. With read float32 [S], w and (optionally) b float32 [C]: returns
+    the layer norm of u = sum_s read[s] new_s, (u - mean) / sqrt(var + eps) *
+    w + b, in out_dtype. One stream with mix = write = read = 1 is the plain
+    residual sum."""
+    T, S, C = streams.shape
+    assert streams.dtype == torch.float32 and streams.is_contiguous()
+    assert (y is None) == (mix is None) == (write is None)
+    assert y2 is None or y is not None
+    assert y2_gate is None or (y2 is not None and y2_gate.dtype == torch.float32
+                               and y2_gate.dim() == 1)
+    assert (read is None) == (w is None) and (y is not None or read is not None)
+    if not streams.is_cuda:
+        return torch_ref.hyper_norm(streams, y, y2, y2_gate, mix, write, read, w, b, eps,
+                                    out_dtype)
+    lib, hip = _lib()
+    for t, n in ((mix, S * S), (write, S), (read, S), (w, C), (b, C)):
+        assert t is None or (t.dtype == torch.float32 and t.is_contiguous() and t.numel() == n)
+    out = torch.empty(T, C, dtype=out_dtype, device=streams.device) if read is not None else None
+    ptr = lambda t: t.data_ptr() if t is not None else None  # noqa: E731
+    rc = lib.oa_hyper_norm(
+        hip.current_stream_ptr(), streams.data_ptr(), S, ptr(y), _rows(y) if y is not None else 0,
+        _dt(y) if y is not None else 1, ptr(y2), _rows(y2) if y2 is not None else 0,
+        _dt(y2) if y2 is not None else 1, ptr(y2_gate),
+        y2_gate.stride(0) if y2_gate is not None else 0, ptr(mix), ptr(write), ptr(read),
+        ptr(w), ptr(b), ptr(out), _dt(out) if out is not None else 1, T, C, float(eps))
+    hip.check(rc, "oa_hyper_norm")
+    return out
+
+
+def rope_rows(x: torch.Tensor, n_rot: int, D: int, inv_freq: torch.Tensor,
+              sb: SeqBatch) -> torch.Tensor:
+    """x [T, n] (may be a column slice): the first n_rot * D columns are heads
+    of D channels whose pairs (2i, 2i+1), i < len(inv_freq), are rotated by
+    position * inv_freq[i] in float32; the other columns are copied. Returns
+    float32 [T, n]: what enters a recurrence stays unrounded."""
+    T, n = x.shape
+    assert n_rot * D <= n and 2 * inv_freq.numel() <= D
+    if not x.is_cuda:
+        return torch_ref.rope_rows(x, n_rot, D, inv_freq, _positions(sb))
+    lib, hip = _lib()
+    assert inv_freq.dtype == torch.float32 and inv_freq.is_contiguous()
+    out = torch.empty(T, n, dtype=torch.float32, device=x.device)
+    rc = lib.oa_rope_rows(
+        hip.current_stream_ptr(), x.data_ptr(), _rows(x), _dt(x), out.data_ptr(), n, n_rot, D,
+        inv_freq.data_ptr(), inv_freq.numel(), sb.seq_of_t.data_ptr(), sb.cu_t.data_ptr(),
+        sb.past_t.data_ptr(), sb.num_seqs, T)
+    hip.check(rc, "oa_rope_rows")
+    return out
+
+
+def combine_norm_gate(a: torch.Tensor, H: int, Dv: int, out_dtype,
+                      a2: Optional[torch.Tensor] = None, lam: float = 0.0, norm: bool = False,
+                      eps: float = 0.0, post_scale: float = 1.0,
+                      gate_logits: Optional[torch.Tensor] = None,
+                      gate_act: str = "sigmoid") -> torch.Tensor:
+    """What follows a mixer's read-out, one launch: o = a - lam * a2 (a2
+    optional; both [T, H*Dv], may be column slices, float32 or bf16); with
+    `norm` each head's Dv values are divided by sqrt(mean(o^2) + eps) and
+    multiplied by post_scale; then o * sigmoid|silu(gate_logits) ([T, H*Dv],
+    may be a column slice; None: no gate). Computed in float32; returns
+    [T, H*Dv] in out_dtype."""
+    T = a.shape[0]
+    assert a.shape[1] == H * Dv and gate_act in ("sigmoid", "silu")
+    assert a2 is None or (a2.shape == a.shape and a2.dtype == a.dtype)
+    if not a.is_cuda:
+        return torch_ref.combine_norm_gate(a, a2, lam, H, Dv, norm, eps, post_scale,
+                                           gate_logits, gate_act, out_dtype)
+    lib, hip = _lib()
+    out = torch.empty(T, H * Dv, dtype=out_dtype, device=a.device)
+    assert gate_logits is None or gate_logits.dtype == out_dtype
+    rc = lib.oa_combine_norm_gate(
+        hip.current_stream_ptr(), a.data_ptr(), _rows(a), _dt(a),
+        a2.data_ptr() if a2 is not None else None, _rows(a2) if a2 is not None else 0,
+        float(lam), gate_logits.data_ptr() if gate_logits is not None else None,
+        _rows(gate_logits) if gate_logits is not None else 0,
+        0 if gate_act == "sigmoid" else 1, out.data_ptr(), _dt(out), T, H, Dv,
+        int(bool(norm)), float(eps), float(post_scale))
+    hip.check(rc, "oa_combine_norm_gate")
+    return out
+
+
+def act_rows(x: torch.Tensor, act: str = "relu2") -> torch.Tensor:
+    """Elementwise activation of an ungated feed-forward on a contiguous
+    buffer: "relu2" (the square of relu), "silu" or "gelu_tanh"; float32
+    inside."""
+    if not x.is_cuda:
+        return torch_ref.act_rows(x, act)
+    lib, hip = _lib()
+    assert x.is_contiguous()
+    out = torch.empty_like(x)
+    hip.check(lib.oa_act_rows(hip.current_stream_ptr(), x.data_ptr(), out.data_ptr(),
+                              x.numel(), _dt(x), ACTS[act]), "oa_act_rows")
+    return out
+
+
+def moe_pairs_plain(x: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor, idx: torch.Tensor,
+                    wts: torch.Tensor, act: str = "relu2") -> torch.Tensor:
+    """Routed ungated experts for few tokens, two launches, no host sync:
+    out[t] = sum_j wts[t,j] * W2[e_tj] act(W1[e_tj] x_t). x [T, K]; w1
+    [E, I, K]; w2 [E, C, I]; idx int32 [T, top]; wts float32 [T, top]. Any
+    sizes, bf16 or float32. A token's result does not depend on the other
+    tokens of the batch."""
+    T, K = x.shape
+    E, I, _ = w1.shape
+    C, top = w2.shape[1], idx.shape[1]
+    if not x.is_cuda:
+        return torch_ref.moe_pairs_plain(x, w1, w2, idx, wts, act)
+    lib, hip = _lib()
+    assert x.is_contiguous() and w1.is_contiguous() and w2.is_contiguous()
+    assert idx.is_contiguous() and idx.dtype == torch.int32
+    assert wts.is_contiguous() and wts.dtype == torch.float32
+    assert w1.dtype == x.dtype and w2.dtype == x.dtype and w2.shape == (E, C, I)
+    mid = torch.empty(T * top, I, dtype=x.dtype, device=x.device)
+    out = torch.empty(T, C, dtype=x.dtype, device=x.device)
+    hip.check(lib.oa_moe_pairs_up(
+        hip.current_stream_ptr(), x.data_ptr(), w1.data_ptr(), idx.data_ptr(), mid.data_ptr(),
+        T, top, E, I, K, _dt(x), ACTS[act]), "oa_moe_pairs_up")
+    hip.check(lib.oa_moe_pairs_down(
+        hip.current_stream_ptr(), mid.data_ptr(), w2.data_ptr(), idx.data_ptr(), wts.data_ptr(),
+        out.data_ptr(), T, top, E, C, I, _dt(x)), "oa_moe_pairs_down")
     return out

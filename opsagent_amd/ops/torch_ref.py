@@ -353,17 +353,20 @@ def dyt_norm(y, post, residual, nxt, out_dtype):
 
 
 def attn_rope_prepare(qkv, q_norm_w, k_norm_w, inv_freq, H, G, D, Dv, eps, k_cache, v_cache,
-                      positions, slot_mapping):
-    """Per-head RMS norm of q and k (weight [D] shared by heads), then rotation
-    of channel pairs (2i, 2i+1), i < len(inv_freq), by position * inv_freq[i];
-    k and v go to their cache slots, q is returned [T, H, D]."""
+                      positions, slot_mapping, v_heads=None):
+    """Per-head RMS norm of q and k (weight [D] shared by heads; None: no
+    norm), then rotation of channel pairs (2i, 2i+1), i < len(inv_freq), by
+    position * inv_freq[i]; k and v (v_heads heads, default G) go to their
+    cache slots, q is returned [T, H, D]."""
     T = qkv.shape[0]
-    x = qkv[:, : H * D + G * D + G * Dv].float()
+    Gv = v_heads or G
+    x = qkv[:, : H * D + G * D + Gv * Dv].float()
     q = x[:, : H * D].reshape(T, H, D)
     k = x[:, H * D : H * D + G * D].reshape(T, G, D)
-    v = x[:, H * D + G * D :].reshape(T, G, Dv)
-    q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_norm_w.float()
-    k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_norm_w.float()
+    v = x[:, H * D + G * D :].reshape(T, Gv, Dv)
+    if q_norm_w is not None:
+        q = q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + eps) * q_norm_w.float()
+        k = k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + eps) * k_norm_w.float()
     r = 2 * inv_freq.numel()
     if r:
         ang = positions.float()[:, None] * inv_freq.float()[None, :]
@@ -380,18 +383,21 @@ def attn_rope_prepare(qkv, q_norm_w, k_norm_w, inv_freq, H, G, D, Dv, eps, k_cac
     nb, bs = k_cache.shape[0], k_cache.shape[1]
     sm = slot_mapping.long()
     k_cache.view(nb * bs, G, D)[sm] = k.to(k_cache.dtype)
-    v_cache.view(nb * bs, G, Dv)[sm] = v.to(v_cache.dtype)
+    v_cache.view(nb * bs, Gv, Dv)[sm] = v.to(v_cache.dtype)
     return q.to(qkv.dtype)
 
 
 def attention_paged(q, k_cache, v_cache, cu, past, block_table, scale, slopes=None,
-                    gate_logits=None, window=None, sinks=None):
+                    gate_logits=None, window=None, sinks=None, softcap=None):
     """Causal softmax attention of each new token over its sequence's cached
     keys. Options: a linear distance penalty slope_h*(i-j), a window (key j
     seen iff i - j < window), a per-head sink term exp(sink_h) in the
-    denominator, a sigmoid gate on each head's output."""
+    denominator, a sigmoid gate on each head's output, a soft cap
+    cap * tanh(score / cap) on the scaled score. The cache may hold fewer
+    value heads than key heads: key head g reads value head g mod Gv."""
     T, H, D = q.shape
-    nb, bs, G, Dv = v_cache.shape
+    nb, bs, Gv, Dv = v_cache.shape
+    G = k_cache.shape[2]
     out = torch.empty(T, H, Dv, dtype=q.dtype, device=q.device)
     rep = H // G
     for b in range(len(cu) - 1):
@@ -405,11 +411,15 @@ def attention_paged(q, k_cache, v_cache, cu, past, block_table, scale, slopes=No
         nblk = (total + bs - 1) // bs
         blocks = block_table[b, fb:nblk].long()
         kk = k_cache[blocks].reshape(-1, G, D)[: total - first].float()
-        vv = v_cache[blocks].reshape(-1, G, Dv)[: total - first].float()
+        vv = v_cache[blocks].reshape(-1, Gv, Dv)[: total - first].float()
+        if Gv != G:
+            vv = vv.repeat(1, G // Gv, 1)
         kk = kk.repeat_interleave(rep, dim=1)
         vv = vv.repeat_interleave(rep, dim=1)
         qs = q[lo:hi].float()
         s = torch.einsum("ihd,jhd->hij", qs, kk) * scale
+        if softcap:
+            s = softcap * torch.tanh(s / softcap)
         i = torch.arange(past[b], total, dtype=torch.float32).view(1, -1, 1)
         j = torch.arange(first, total, dtype=torch.float32).view(1, 1, -1)
         if slopes is not None:
@@ -587,3 +597,89 @@ def gated_rms_norm(o, w, groups, gate_logits, gate_act, eps, out_dtype):
     g = gate_logits.float()
     g = torch.sigmoid(g) if gate_act == "sigmoid" else torch.nn.functional.silu(g)
     return (x * g).to(out_dtype)
+
+
+# ---------------------------------------------------------------------------
+# Hyper-connected pre-norm decoders: several residual streams, differential
+# attention, retention, ungated experts.
+
+
+def hyper_norm(streams, y, y2, y2_gate, mix, write, read, w, b, eps, out_dtype):
+    """streams float32 [T, S, C], updated in place. With y (and mix [S, S]
+    indexed [from, to], write [S]): new_t = sum_s mix[s, t] old_s + write[t] *
+    (y + sigmoid(y2_gate) * y2), every stream from the OLD ones. With read
+    [S]: returns the layer norm ((u - mean) / sqrt(var + eps) * w + b) of
+    u = sum_s read[s] new_s in out_dtype."""
+    if y is not None:
+        yy = y.float()
+        if y2 is not None:
+            g = torch.sigmoid(y2_gate.float()).unsqueeze(-1) if y2_gate is not None else 1.0
+            yy = yy + g * y2.float()
+        new = (torch.einsum("sb,asc->abc", mix.float(), streams)
+               + write.float().view(1, -1, 1) * yy.unsqueeze(1))
+        streams.copy_(new)
+    if read is None:
+        return None
+    u = torch.einsum("s,tsc->tc", read.float(), streams)
+    mu = u.mean(-1, keepdim=True)
+    d = u - mu
+    out = d * torch.rsqrt(d.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+    if b is not None:
+        out = out + b.float()
+    return out.to(out_dtype)
+
+
+def rope_rows(x, n_rot, D, inv_freq, pos):
+    """x [T, n]: the first n_rot * D columns are heads of D channels whose
+    pairs (2i, 2i+1), i < len(inv_freq), turn by pos * inv_freq[i]; the other
+    columns are copied. Returns float32 [T, n]."""
+    T = x.shape[0]
+    out = x.float().clone()
+    if inv_freq.numel():
+        out[:, : n_rot * D] = _rotate_pairs(out[:, : n_rot * D].reshape(T, n_rot, D), pos,
+                                            inv_freq).reshape(T, n_rot * D)
+    return out
+
+
+def combine_norm_gate(a, a2, lam, H, Dv, norm, eps, post_scale, gate_logits, gate_act, out_dtype):
+    """a [T, H*Dv] (minus lam * a2 if a2 is given); with norm each head's Dv
+    values are divided by their root mean square (eps inside the root) and
+    multiplied by post_scale; then times sigmoid or silu of gate_logits
+    [T, H*Dv] (None: no gate)."""
+    T = a.shape[0]
+    o = a.float()
+    if a2 is not None:
+        o = o - float(lam) * a2.float()
+    if norm:
+        o = o.view(T, H, Dv)
+        o = (o * torch.rsqrt(o.pow(2).mean(-1, keepdim=True) + eps) * post_scale).reshape(T, H * Dv)
+    if gate_logits is not None:
+        g = gate_logits.float()
+        o = o * (torch.sigmoid(g) if gate_act == "sigmoid" else torch.nn.functional.silu(g))
+    return o.to(out_dtype)
+
+
+def act_rows(x, act):
+    """Elementwise activation of an ungated feed-forward: "relu2" (the square
+    of relu), "silu", "gelu_tanh"; evaluated in float32."""
+    z = x.float()
+    if act == "relu2":
+        z = torch.relu(z).square()
+    elif act == "silu":
+        z = torch.nn.functional.silu(z)
+    else:
+        z = gelu_tanh(z)
+    return z.to(x.dtype)
+
+
+def moe_pairs_plain(x, w1, w2, idx, wts, act):
+    """out[t] = sum_j wts[t, j] * W2[e] act(W1[e] x_t), e = idx[t, j]; w1
+    [E, I, K], w2 [E, C, I]."""
+    T, top = idx.shape
+    out = torch.zeros(T, w2.shape[1], dtype=torch.float32, device=x.device)
+    for t in range(T):
+        for j in range(top):
+            e = int(idx[t, j])
+            a = act_rows(torch.nn.functional.linear(x[t : t + 1], w1[e]), act)
+            out[t] += wts[t, j] * torch.nn.functional.linear(a, w2[e])[0].float()
+    return out.to(x.dtype)
