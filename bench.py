@@ -83,7 +83,7 @@ def main() -> None:
     ap.add_argument("--mode", choices=["turn", "multiturn", "concurrent", "layers"],
                     default="turn",
                     help="layers: prefill/decode throughput of the hybrid decoders "
-                         "(Povazen, Vazilorn, Rafodra) beside llama / llama-moe layers of equal "
+                         "(Povazen, Vazilorn, Rafodra, Suzulix) beside llama / llama-moe layers of equal "
                          "size (extra mode; prints one JSON line per size and batch)")
     ap.add_argument("--layer-models", default="llama,povazen",
                     help="layers mode: which models to run (llama, povazen, llama-moe, "

@@ -873,6 +873,19 @@ HYBRID_REGISTRY = {
         kv_rank=128, q_rank=256, rot_dim=32, lat_dim=64, lat_vdim=64, ret_heads=8,
         ret_dim=128, ret_vdim=128, experts=16, top=4, expert_ff=512, shared_ff=512,
         streams=2, loop=(0, 2, 2), embed_scale=8.0, logit_scale=0.25),
+    # layer shapes of ~1B- and ~8B-class models at 4 layers (speed beside
+    # Rafodra layers of equal width): two maps of half a head each, a 192 + 64
+    # wide cached latent, 16 experts of ff/8 with 4 per token
+    "suzulix-4l2k": lambda: suzulix_config_dict(
+        vocab=2048, width=2048, pattern="LmAmRmRm", heads=16, kv_heads=4, dim=64, vdim=128,
+        kv_rank=192, q_rank=512, rot_dim=64, lat_dim=128, lat_vdim=128, rot_base=500000.0,
+        ret_heads=16, ret_dim=128, ret_vdim=128, experts=16, top=4, expert_ff=1024,
+        shared_ff=1024, streams=2),
+    "suzulix-4l4k": lambda: suzulix_config_dict(
+        vocab=2048, width=4096, pattern="LmAmRmRm", heads=32, kv_heads=8, dim=64, vdim=128,
+        kv_rank=192, q_rank=1024, rot_dim=64, lat_dim=128, lat_vdim=128, rot_base=500000.0,
+        ret_heads=32, ret_dim=128, ret_vdim=128, experts=16, top=4, expert_ff=1792,
+        shared_ff=1792, streams=2),
 }
 
 

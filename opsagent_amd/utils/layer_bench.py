@@ -22,6 +22,8 @@ from opsagent_amd.engine.config import (
     povazen_spec_from_dict,
     rafodra_config_dict,
     rafodra_spec_from_dict,
+    suzulix_config_dict,
+    suzulix_spec_from_dict,
     vazilorn_config_dict,
     vazilorn_spec_from_dict,
 )
@@ -77,7 +79,25 @@ def specs_for(size) -> Dict[str, object]:
             name=f"rafodra-{tag}-{name}",
         )
 
+    def sz(pattern, streams, tag):
+        # latent attention, differential attention (two maps of half a head
+        # each: llama's query/key width), retention twice; the cached latent
+        # and the routed feed-forwards have Rafodra's shapes (experts ungated)
+        return suzulix_spec_from_dict(
+            suzulix_config_dict(vocab=32000, width=width, pattern=(pattern * layers)[:2 * layers],
+                                heads=heads, kv_heads=kv, dim=dim // 2, vdim=dim, kv_rank=192,
+                                q_rank=width // 4, rot_dim=64, lat_dim=dim, lat_vdim=dim,
+                                rot_base=500000.0, ret_heads=heads, ret_dim=dim, ret_vdim=dim,
+                                experts=experts, top=top, expert_ff=eff, shared_ff=eff,
+                                streams=streams),
+            name=f"suzulix-{tag}-{name}",
+        )
+
     return {
+        "suzulix": sz("LmAmRmRm", 2, "moe"),
+        # mixers alone (no feed-forward) beside Rafodra's: what the streams,
+        # the two maps and the rotation cost without the experts
+        "suzulix-mix": sz("L-A-R-R-", 2, "mix"), "rafodra-mix": rf("L-G-A-S-", "mix"),
         "llama": llama, "povazen": hybrid, "llama-moe": llama_moe,
         "rafodra": rf("LdGdAdSd", "dense"), "rafodra-moe": rf("LmGmAmSm", "moe"),
         # a window wider than the prompt: the attention kernels do llama's work
@@ -90,7 +110,8 @@ def specs_for(size) -> Dict[str, object]:
 
 # which model each one is measured against
 BASELINE_OF = {"povazen": "llama", "vazilorn": "llama", "vazilorn-w512": "llama",
-               "vazilorn-moe": "llama-moe", "rafodra": "povazen", "rafodra-moe": "vazilorn-moe"}
+               "vazilorn-moe": "llama-moe", "rafodra": "povazen", "rafodra-moe": "vazilorn-moe",
+               "suzulix": "rafodra-moe", "suzulix-mix": "rafodra-mix"}
 
 
 def _run(spec, batch: int, prompt: int, decode: int, reps: int) -> Dict[str, float]:

@@ -1,0 +1,765 @@
+"""The Suzulix decoder in the framework (engine, paged cache, state slots,
+scheduler, ops/kernels) against the plain oracle in suzulix_oracle.py.
+
+Unmarked cases run on the CPU path (float32); gpu-marked cases run the HIP
+kernels in float32 and bfloat16. Configurations are small and irregular:
+sizes that are not powers of two, key size != value size, three residual
+streams, a looped run of layers, layers without a feed-forward.
+"""
+
+import copy
+import json
+import math
+
+import pytest
+import torch
+
+import suzulix_oracle as O
+from opsagent_amd.engine.config import suzulix_config_dict, suzulix_spec_from_dict
+from opsagent_amd.engine.engine import LLMEngine, SamplingParams
+from opsagent_amd.engine.replay import TraceReplayer
+from opsagent_amd.ops import mixer_ops as mx
+
+gpu = pytest.mark.gpu
+MODES = [
+    pytest.param(("cpu", "fp32"), id="cpu-f32"),
+    pytest.param(("cuda", "fp32"), id="gpu-f32", marks=gpu),
+    pytest.param(("cuda", "bf16"), id="gpu-bf16", marks=gpu),
+]
+F64 = torch.float64
+
+
+def _skip_if_wrong_device(device):
+    if device == "cpu" and torch.cuda.is_available():
+        pytest.skip("the engine picks the GPU on this box; CPU path is covered on CPU runs")
+
+
+def tdtype(name):
+    return torch.float32 if name == "fp32" else torch.bfloat16
+
+
+def close(got, want, dtype, what="", loose=1.0):
+    got, want = got.detach().double().cpu(), want.detach().double().cpu()
+    assert got.shape == want.shape, (got.shape, want.shape)
+    err = (got - want).pow(2).mean().sqrt() / (want.pow(2).mean().sqrt() + 1e-9)
+    worst = (got - want).abs().max() / (want.abs().max() + 1e-9)
+    if dtype == "fp32":
+        assert err < 1e-4 * loose and worst < 1e-3 * loose, f"{what}: rel rms {err:.3e}, worst {worst:.3e}"
+    else:
+        assert err < 3e-2 * loose and worst < 1.5e-1 * loose, f"{what}: rel rms {err:.3e}, worst {worst:.3e}"
+
+
+def make_cfg(pattern="LmAmRmR-Am", width=40, vocab=97, **kw):
+    base = dict(heads=6, kv_heads=2, dim=12, vdim=10, kv_rank=18, q_rank=22, rot_dim=6,
+                lat_heads=3, lat_dim=8, lat_vdim=14, rot_dims=8, rot_base=50.0, scale=0.23,
+                softcap=4.0, diff=0.3, ret_heads=2, ret_dim=20, ret_vdim=12, ret_rot_dims=12,
+                decay=[0.7, 0.995], experts=12, top=3, expert_ff=20, shared_ff=28, streams=3,
+                loop=(1, 3, 2), embed_scale=3.0, logit_scale=0.4, eps=1e-5)
+    base.update(kw)
+    return suzulix_config_dict(vocab, width, pattern, **base)
+
+
+def x16_cfg(pattern="LmAmRmR-Am"):
+    """Sizes the matrix-core attention kernel and the vector paths take."""
+    return make_cfg(pattern, width=64, heads=4, kv_heads=2, dim=32, vdim=16, kv_rank=32, q_rank=48,
+                    rot_dim=16, lat_heads=4, lat_dim=16, lat_vdim=16, rot_dims=16, ret_heads=4,
+                    ret_dim=32, ret_vdim=32, ret_rot_dims=32, decay=[0.6, 0.9, 0.97, 0.999],
+                    expert_ff=32, shared_ff=48, streams=2)
+
+
+def rounded(W, dtype):
+    """The oracle sees the weights the engine holds (bfloat16-rounded in bf16 mode)."""
+    if dtype == "bf16":
+        return {k: v.to(torch.bfloat16).float() for k, v in W.items()}
+    return W
+
+
+def build_engine(cfg, W, dtype="fp32", blocks=64, block_size=8, slots=4, **extra):
+    eng = LLMEngine(dict({
+        "model": suzulix_spec_from_dict(cfg), "dtype": dtype, "kv_num_blocks": blocks,
+        "kv_block_size": block_size, "max_batch_size": slots, "state_slots": slots,
+        "tokenizer_check": False, "max_seq_len": 4096, "max_prefill_chunk": 4096,
+    }, **extra))
+    eng.model.load_named_tensors(rounded(W, dtype))
+    return eng
+
+
+def tokens_for(cfg, n, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, cfg["vocab"], (n,), generator=g).tolist()
+
+
+def replay(eng, schedule):
+    """schedule: list of steps; step = list of (id, tokens, last?) -> id -> logits of every position."""
+    rp = TraceReplayer(eng)
+    got = {}
+    for step in schedule:
+        entries = [{"id": i, "tokens": t, "want": list(range(len(t)))} for i, t, _ in step]
+        end = [i for i, _, last in step if last]
+        out = rp.step(entries, end)
+        off = 0
+        for i, t, _ in step:
+            got.setdefault(i, []).append(out[off:off + len(t)])
+            off += len(t)
+    return {i: torch.cat(v, 0) for i, v in got.items()}
+
+
+def cut(tokens, sizes):
+    out, at, k = [], 0, 0
+    while at < len(tokens):
+        n = sizes[k % len(sizes)]
+        out.append(tokens[at:at + n])
+        at += n
+        k += 1
+    return out
+
+
+def dev_of(device):
+    return "cuda" if device == "cuda" else "cpu"
+
+
+# --------------------------------------------------------------------------
+# mechanisms alone
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("S", [1, 2, 3, 5])
+@pytest.mark.parametrize("C", [24, 7, 4100])
+def test_stream_write_read_norm(mode, S, C):
+    """x_t <- sum_s mix[s, t] x_s + out[t] (y + sigmoid(g) y2), all streams from
+    the old ones; then the biased layer norm of sum_s in[s] x_s. Also each half
+    alone, and rows wider than the kernel keeps in registers."""
+    device, dtype = mode
+    _skip_if_wrong_device(device)
+    dev, dt = dev_of(device), tdtype(dtype)
+    g = torch.Generator().manual_seed(100 * S + C)
+    T = 4
+    xs = (2.0 + torch.randn(T, S, C, generator=g)).to(dev)
+    y = torch.randn(T, C + 3, generator=g).to(dt).to(dev)[:, 2:C + 2]
+    y2 = torch.randn(T, C, generator=g).to(dt).to(dev)
+    gate = torch.randn(T, 3, generator=g).to(dev)[:, 1]
+    mix = (torch.eye(S) + 0.4 * torch.randn(S, S, generator=g)).to(dev)       # not symmetric
+    wr, rd = torch.randn(S, generator=g).to(dev), torch.randn(S, generator=g).to(dev)
+    w, b = (1.0 + 0.3 * torch.randn(C, generator=g)).to(dev), torch.randn(C, generator=g).to(dev)
+    eps = 1e-5
+
+    def want(x, with_y, with_y2, with_read):
+        x = x.double().cpu()
+        if with_y:
+            yy = y.double().cpu()
+            if with_y2:
+                yy = yy + O.sigmoid(gate.double().cpu()).unsqueeze(1) * y2.double().cpu()
+            x = torch.stack([sum(mix[s, t].double().cpu() * x[:, s] for s in range(S))
+                             + wr[t].double().cpu() * yy for t in range(S)], 1)
+        out = None
+        if with_read:
+            u = sum(rd[s].double().cpu() * x[:, s] for s in range(S))
+            out = O.layer_norm(u, w.double().cpu(), b.double().cpu(), eps)
+        return x, out
+
+    for with_y, with_y2, with_read in [(True, True, True), (True, False, True), (False, False, True),
+                                       (True, True, False)]:
+        x = xs.clone()
+        got = mx.hyper_norm(x, rd if with_read else None, w if with_read else None,
+                            b if with_read else None, eps, dt,
+                            y=y if with_y else None, mix=mix if with_y else None,
+                            write=wr if with_y else None, y2=y2 if with_y2 else None,
+                            y2_gate=gate if with_y2 else None)
+        wx, wo = want(xs, with_y, with_y2, with_read)
+        close(x, wx, "fp32", "streams", loose=1.0 if dtype == "fp32" else 10.0)
+        if with_read:
+            close(got, wo, dtype, "normed read")
+        else:
+            assert got is None
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("geom", [(5, 12, 8, 7), (4, 16, 16, 0), (3, 6, 2, 33), (2, 64, 64, 64)])
+def test_rows_rotated_into_float32(mode, geom):
+    """Rotated heads beside copied columns, from a column slice, at positions
+    that continue two sequences."""
+    device, dtype = mode
+    _skip_if_wrong_device(device)
+    dev, dt = dev_of(device), tdtype(dtype)
+    n_rot, D, dims, rest = geom
+    g = torch.Generator().manual_seed(sum(geom))
+    sb = mx.SeqBatch.build([(37, 3, 0, list(range(8))), (0, 4, 1, list(range(8, 10)))], 8, dev)
+    T = 7
+    x = torch.randn(T, n_rot * D + rest + 5, generator=g).to(dt).to(dev)[:, 3:3 + n_rot * D + rest]
+    inv = mx.rotary_inv_freq(dims, 300.0).to(dev)
+    got = mx.rope_rows(x, n_rot, D, inv, sb)
+    assert got.dtype == torch.float32
+    pos = torch.tensor([37, 38, 39, 0, 1, 2, 3])
+    xd = x.double().cpu()
+    want = xd.clone()
+    for h in range(n_rot):
+        want[:, h * D:(h + 1) * D] = O.turn(xd[:, h * D:(h + 1) * D], pos, dims, 300.0, "interleaved")
+    close(got, want, "fp32", "rotated rows")
+
+
+def test_half_layout_rows_reordered_keep_every_product():
+    """Rows taken from the "half" pairing to the interleaved one, rotated as
+    interleaved pairs, give the dot products of the half-layout rotation."""
+    from opsagent_amd.engine.hybrid import _relayout_heads
+
+    g = torch.Generator().manual_seed(5)
+    H, D, off, dims, C = 3, 14, 4, 8, 9
+    wq, wk = torch.randn(H * D, C, generator=g).double(), torch.randn(H * D, C, generator=g).double()
+    x = torch.randn(6, C, generator=g).double()
+    pos = torch.tensor([0, 1, 5, 17, 100, 1000])
+
+    def products(wq_, wk_, layout):
+        q, k = (x @ wq_.T).reshape(6, H, D), (x @ wk_.T).reshape(6, H, D)
+        out = []
+        for h in range(H):
+            qq, kk = q[:, h].clone(), k[:, h].clone()
+            qq[:, off:] = O.turn(q[:, h, off:], pos, dims, 77.0, layout)
+            kk[:, off:] = O.turn(k[:, h, off:], pos, dims, 77.0, layout)
+            out.append(qq @ kk.T)
+        return torch.stack(out)
+
+    want = products(wq, wk, "half")
+    got = products(_relayout_heads(wq, H, D, off, dims, "half"),
+                   _relayout_heads(wk, H, D, off, dims, "half"), "interleaved")
+    assert torch.allclose(got, want, atol=1e-12)
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("case", [(3, 10, True, True, "sigmoid"), (4, 16, True, False, "silu"),
+                                  (2, 300, True, True, "sigmoid"), (5, 7, False, False, "sigmoid"),
+                                  (1, 32, False, True, "silu")])
+def test_combine_head_norm_gate(mode, case):
+    device, dtype = mode
+    _skip_if_wrong_device(device)
+    dev, dt = dev_of(device), tdtype(dtype)
+    H, Dv, norm, two, act = case
+    g = torch.Generator().manual_seed(H * Dv)
+    T, n = 5, H * Dv
+    both = (3.0 * torch.randn(T, 2 * n, generator=g)).to(dt).to(dev)
+    gate = torch.randn(T, n + 2, generator=g).to(dt).to(dev)[:, 2:]
+    lam, eps, post = 0.37, 1e-5, 0.7
+    got = mx.combine_norm_gate(both[:, :n], H, Dv, dt, a2=both[:, n:] if two else None, lam=lam,
+                               norm=norm, eps=eps, post_scale=post, gate_logits=gate, gate_act=act)
+    o = both[:, :n].double().cpu()
+    if two:
+        o = o - lam * both[:, n:].double().cpu()
+    if norm:
+        o = (O.unit_rms(o.reshape(T, H, Dv), eps) * post).reshape(T, n)
+    z = gate.double().cpu()
+    o = o * (O.sigmoid(z) if act == "sigmoid" else z * O.sigmoid(z))
+    close(got, o, dtype, "combine")
+    # float32 read-out into the model's type (the recurrent mixers' case)
+    a32 = both[:, :n].float()
+    got = mx.combine_norm_gate(a32, H, Dv, dt, norm=True, eps=eps, gate_logits=gate, gate_act="silu")
+    o = O.unit_rms(a32.double().cpu().reshape(T, H, Dv), eps).reshape(T, n) * (z * O.sigmoid(z))
+    close(got, o, dtype, "combine from float32")
+
+
+def _attend(mode, H, G, Gv, D, Dv, past, n, q, keys, vals, scale, cap, block_size=8):
+    """Run attention_paged for ONE sequence whose cache rows are given whole
+    (keys [total, G, D], vals [total, Gv, Dv]); q [n, H, D]."""
+    device, dtype = mode
+    dev, dt = dev_of(device), tdtype(dtype)
+    total = past + n
+    nblk = (total + block_size - 1) // block_size
+    order = list(range(nblk + 2, 2, -1))                    # pages in falling order
+    kc = torch.zeros(nblk + 4, block_size, G, D, dtype=dt, device=dev)
+    vc = torch.zeros(nblk + 4, block_size, Gv, Dv, dtype=dt, device=dev)
+    for j in range(total):
+        kc[order[j // block_size], j % block_size] = keys[j].to(dt).to(dev)
+        vc[order[j // block_size], j % block_size] = vals[j].to(dt).to(dev)
+    sb = mx.SeqBatch.build([(past, n, 0, order)], block_size, dev)
+    return mx.attention_paged(q.to(dt).to(dev).contiguous(), kc, vc, sb, scale, softcap=cap)
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("back", [0, 1, 7, 8, 63, 64, 65, 300, 511])
+@pytest.mark.parametrize("decode", [False, True])
+def test_far_key_stands_out_under_the_cap(mode, back, decode):
+    """One key `back` positions behind the last query carries a large product
+    with it; its value must dominate the output, in a prompt portion and for a
+    single decoded token, with two key heads per value head and a soft cap."""
+    device, dtype = mode
+    _skip_if_wrong_device(device)
+    H, G, Gv, D, Dv = 4, 2, 1, 16, 16
+    total = 520
+    n = 1 if decode else 9
+    past = total - n
+    g = torch.Generator().manual_seed(back)
+    keys = 0.05 * torch.randn(total, G, D, generator=g)
+    vals = torch.randn(total, Gv, Dv, generator=g)
+    q = 0.05 * torch.randn(n, H, D, generator=g)
+    target = total - 1 - back
+    keys[target, :, 0] = 6.0
+    q[-1, :, 0] = 6.0
+    scale, cap = 0.5, 12.0
+    got = _attend(mode, H, G, Gv, D, Dv, past, n, q, keys, vals, scale, cap)
+    dt = tdtype(dtype)
+    qd, kd, vd = (t.to(dt).double() for t in (q, keys, vals))
+    want = torch.zeros(n, H, Dv, dtype=F64)
+    for i in range(n):
+        for h in range(H):
+            s = kd[: past + i + 1, h // (H // G)] @ qd[i, h] * scale
+            s = cap * torch.tanh(s / cap)
+            p = torch.softmax(s, 0)
+            want[i, h] = p @ vd[: past + i + 1, 0]
+    close(got.reshape(n, H, Dv), want, dtype, f"key {back} back")
+    # the far key holds nearly all the weight of the last query
+    assert (got.reshape(n, H, Dv)[-1].double().cpu() - vd[target, 0]).abs().max() < 0.2
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_soft_cap_saturates(mode):
+    """Scores far above the cap are all worth the cap: two keys whose raw
+    scores differ by a factor of two share the weight almost evenly, which no
+    uncapped softmax would do."""
+    device, dtype = mode
+    _skip_if_wrong_device(device)
+    H, G, Gv, D, Dv = 2, 2, 2, 16, 16
+    keys = torch.zeros(3, G, D)
+    keys[0, :, 0], keys[1, :, 0], keys[2, :, 0] = 8.0, 16.0, -8.0
+    vals = torch.zeros(3, Gv, Dv)
+    vals[0, :, 0], vals[1, :, 1], vals[2, :, 2] = 1.0, 1.0, 1.0
+    q = torch.zeros(1, H, D)
+    q[0, :, 0] = 4.0
+    out = _attend(mode, H, G, Gv, D, Dv, 2, 1, q, keys, vals, 1.0, 3.0).reshape(H, Dv).double().cpu()
+    e = math.exp(-6.0)                                   # the key at -cap against two at +cap
+    assert abs(float(out[0, 0]) - 1 / (2 + e)) < 2e-2 and abs(float(out[0, 1]) - 1 / (2 + e)) < 2e-2
+    plain = _attend(mode, H, G, Gv, D, Dv, 2, 1, q, keys, vals, 1.0, None).reshape(H, Dv)
+    assert float(plain[0, 1]) > 0.99
+
+
+MIXER_GEOMS = {
+    "L": [dict(lat_heads=3, lat_dim=8, lat_vdim=14, kv_rank=18, q_rank=22, rot_dim=6),
+          dict(lat_heads=4, lat_dim=16, lat_vdim=16, kv_rank=32, q_rank=16, rot_dim=16),
+          dict(lat_heads=1, lat_dim=4, lat_vdim=5, kv_rank=9, q_rank=3, rot_dim=2),
+          dict(lat_heads=2, lat_dim=8, lat_vdim=40, kv_rank=64, q_rank=64, rot_dim=32)],
+    "A": [dict(heads=6, kv_heads=2, dim=12, vdim=10, rot_dims=8),
+          dict(heads=4, kv_heads=2, dim=32, vdim=16, rot_dims=32),
+          dict(heads=2, kv_heads=2, dim=16, vdim=32, rot_dims=0, softcap=None),
+          dict(heads=3, kv_heads=1, dim=7, vdim=5, rot_dims=6, diff=0.8),
+          dict(heads=32, kv_heads=1, dim=16, vdim=16, rot_dims=4)],
+    "R": [dict(ret_heads=2, ret_dim=20, ret_vdim=12, ret_rot_dims=12),
+          dict(ret_heads=4, ret_dim=32, ret_vdim=32, ret_rot_dims=32, decay=[0.6, 0.9, 0.97, 0.999]),
+          dict(ret_heads=1, ret_dim=7, ret_vdim=5, ret_rot_dims=0, decay=[0.5]),
+          dict(ret_heads=2, ret_dim=130, ret_vdim=36, ret_rot_dims=64)],
+}
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("kind,k", [(kind, k) for kind in "LAR" for k in range(len(MIXER_GEOMS[kind]))])
+def test_mixer_alone(mode, kind, k):
+    """One layer without a feed-forward on one plain residual stream: the
+    residual after it is embedding + mixer(norm(embedding)); read in two
+    portions so that the second continues cache or state."""
+    device, dtype = mode
+    _skip_if_wrong_device(device)
+    cfg = make_cfg(kind + "-", streams=None, loop=None, **MIXER_GEOMS[kind][k])
+    W = O.random_weights(cfg, seed=3 + k)
+    eng = build_engine(cfg, W, dtype)
+    toks = tokens_for(cfg, 29, k)
+    layers = []
+    O.forward(cfg, rounded(W, dtype), toks, layers)
+    eng.model.trace_layers = []
+    replay(eng, [[("a", toks[:17], False)], [("a", toks[17:], True)]])
+    got = torch.cat(eng.model.trace_layers, 0)
+    close(got, layers[0], dtype, f"{kind} geometry {k}")
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_slow_decay_remembers_the_first_token(mode):
+    """With decay 1 - 2^-14 a head still reads the first token after hundreds
+    of steps; the other head (decay 0.5) has long forgotten it. The logits at
+    the end depend on the first token only through the slow head."""
+    device, dtype = mode
+    _skip_if_wrong_device(device)
+    cfg = make_cfg("R-", streams=None, loop=None, decay=[1.0 - 2.0 ** -14, 0.5])
+    W = O.random_weights(cfg, seed=4)
+    eng = build_engine(cfg, W, dtype)
+    toks = tokens_for(cfg, 400, 6)
+    other = [(toks[0] + 1) % cfg["vocab"]] + toks[1:]
+    Wr = rounded(W, dtype)
+    want = O.forward(cfg, Wr, toks)[-3:]
+    assert (want - O.forward(cfg, Wr, other)[-3:]).abs().max() > 1e-3
+    parts = [toks[:200], toks[200:397]] + [[t] for t in toks[397:]]
+    got = replay(eng, [[("a", p, k == len(parts) - 1)] for k, p in enumerate(parts)])["a"][-3:]
+    close(got, want, dtype, "after 400 tokens")
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("sizes", [(40, 20, 28, 12, 3), (64, 32, 0, 8, 2), (24, 9, 7, 5, 5), (32, 16, 16, 4, 1)])
+def test_ungated_experts_paths(mode, sizes):
+    """Few-token pair kernels and the sorted per-expert path against the
+    oracle: biased router, weights from the chosen logits only, gated shared
+    expert."""
+    device, dtype = mode
+    _skip_if_wrong_device(device)
+    C, ff, shared, experts, top = sizes
+    cfg = make_cfg("R-Rm", width=C, streams=None, loop=None, experts=experts, top=top, expert_ff=ff,
+                   shared_ff=shared)
+    W = O.random_weights(cfg, seed=sum(sizes))
+    eng = build_engine(cfg, W, dtype)
+    mlp = eng.model.layers[1].mlp
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(37, C, generator=g).to(tdtype(dtype))
+    Wd = {k: v.double() for k, v in rounded(W, dtype).items()}
+    want = O.moe_ff(x.double(), Wd, "l1.mlp.", cfg["layers"][1]["mlp"])
+    for path in ("pairs", "sorted"):
+        mlp.force_path = path
+        close(mlp(x.to(eng.device)), want, dtype, path, loose=2.0)
+    mlp.force_path = None
+    close(mlp(x[:3].to(eng.device)), want[:3], dtype, "default path", loose=2.0)
+
+
+@pytest.mark.parametrize("mode", MODES[:2])
+def test_router_bias_alone_chooses(mode):
+    """With a zero router matrix the bias alone ranks the experts, and the
+    weights are the softmax over the chosen biases only."""
+    device, dtype = mode
+    _skip_if_wrong_device(device)
+    cfg = make_cfg("Rm", streams=None, loop=None, experts=7, top=3, shared_ff=0)
+    W = O.random_weights(cfg, seed=2)
+    W["l0.mlp.router"] = torch.zeros_like(W["l0.mlp.router"])
+    W["l0.mlp.router.b"] = torch.tensor([0.1, 2.0, -1.0, 1.5, 0.0, 1.9, -3.0])
+    eng = build_engine(cfg, W, dtype)
+    idx, wts = eng.model.layers[0].mlp.route(torch.randn(5, cfg["width"]).to(eng.device))
+    assert idx.cpu().tolist() == [[1, 5, 3]] * 5
+    want = torch.softmax(torch.tensor([2.0, 1.9, 1.5]), 0)
+    assert torch.allclose(wts.cpu(), want.expand(5, 3), atol=1e-6)
+
+
+# --------------------------------------------------------------------------
+# whole models
+
+
+@pytest.fixture(scope="module", params=["odd", "x16"])
+def model_case(request):
+    cfg = make_cfg() if request.param == "odd" else x16_cfg()
+    return cfg, O.random_weights(cfg, seed=1)
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_layers_and_logits_whole_prompt(mode, model_case):
+    device, dtype = mode
+    _skip_if_wrong_device(device)
+    cfg, W = model_case
+    eng = build_engine(cfg, W, dtype)
+    toks = tokens_for(cfg, 45, 2)
+    layers = []
+    want = O.forward(cfg, rounded(W, dtype), toks, layers)
+    eng.model.trace_layers = []
+    got = replay(eng, [[("a", toks, True)]])["a"]
+    assert len(eng.model.trace_layers) == len(layers) == 7      # two looped layers count twice
+    for i, x in enumerate(eng.model.trace_layers):
+        close(x, layers[i], dtype, f"sum of streams after run {i}")
+    close(got, want, dtype, "logits")
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_first_tokens(mode, model_case):
+    device, dtype = mode
+    _skip_if_wrong_device(device)
+    cfg, W = model_case
+    eng = build_engine(cfg, W, dtype)
+    Wr = rounded(W, dtype)
+    for n in (1, 2, 3):
+        toks = tokens_for(cfg, n, 10 + n)
+        want = O.forward(cfg, Wr, toks)
+        close(replay(eng, [[("s", toks, True)]])["s"], want, dtype, f"{n} tokens at once")
+        close(replay(eng, [[("s", [t], k == n - 1)] for k, t in enumerate(toks)])["s"], want, dtype,
+              f"{n} tokens one by one")
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("sizes", [[1], [2], [3, 2], [7, 1, 2], [8], [16, 5], [9, 1, 1, 30]])
+def test_portions_and_decode(mode, model_case, sizes):
+    """Any cut of the prompt, token-by-token decoding included, gives the
+    logits of the whole prompt at once."""
+    device, dtype = mode
+    _skip_if_wrong_device(device)
+    cfg, W = model_case
+    eng = build_engine(cfg, W, dtype)
+    toks = tokens_for(cfg, 61, 3)
+    want = O.forward(cfg, rounded(W, dtype), toks)
+    parts = cut(toks, sizes)
+    got = replay(eng, [[("a", p, k == len(parts) - 1)] for k, p in enumerate(parts)])["a"]
+    close(got, want, dtype, f"portions {sizes}")
+    assert eng.kv.num_free() == eng.kv.num_blocks and eng.state_pool.num_free() == 4
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_unequal_batch_equals_alone(mode, model_case):
+    """Four unequal requests share steps (portions beside single tokens, one
+    sitting out now and then); each equals itself alone."""
+    device, dtype = mode
+    _skip_if_wrong_device(device)
+    cfg, W = model_case
+    eng = build_engine(cfg, W, dtype)
+    Wr = rounded(W, dtype)
+    reqs = {"a": tokens_for(cfg, 53, 4), "b": tokens_for(cfg, 9, 5), "c": tokens_for(cfg, 1, 7),
+            "d": tokens_for(cfg, 30, 7)}
+    plan = {"a": cut(reqs["a"], [11, 2, 1, 1, 19]), "b": cut(reqs["b"], [1]),
+            "c": [reqs["c"]], "d": cut(reqs["d"], [2, 13, 1])}
+    schedule, k = [], 0
+    while any(plan.values()):
+        step = []
+        for i in sorted(plan):
+            if plan[i] and not (i == "a" and k % 4 == 3):
+                p = plan[i].pop(0)
+                step.append((i, p, not plan[i]))
+        schedule.append(step)
+        k += 1
+    got = replay(eng, schedule)
+    for i, toks in reqs.items():
+        close(got[i], O.forward(cfg, Wr, toks), dtype, f"request {i} in a mixed batch")
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_pages_and_slots_used_again(mode, model_case):
+    """A pool of 6 pages and 2 slots serves 7 requests in turn; freed pages
+    come back in another order and hold stale keys, freed slots stale state
+    (of every pass of the looped layers)."""
+    device, dtype = mode
+    _skip_if_wrong_device(device)
+    cfg, W = model_case
+    eng = build_engine(cfg, W, dtype, blocks=6, block_size=8, slots=2)
+    Wr = rounded(W, dtype)
+    lens = [20, 17, 25, 3, 24, 9, 22]
+    reqs = {"r%d" % k: tokens_for(cfg, n, 20 + k) for k, n in enumerate(lens)}
+    rp = TraceReplayer(eng)
+    names = list(reqs)
+    live, nxt, got = {}, 0, {i: [] for i in reqs}
+    while nxt < len(names) or live:
+        while nxt < len(names) and len(live) < 2:
+            need = sum((len(reqs[i]) + 7) // 8 for i in live) + (len(reqs[names[nxt]]) + 7) // 8
+            if need > 6:
+                break
+            live[names[nxt]] = cut(reqs[names[nxt]], [5, 1, 2, 7])
+            nxt += 1
+        entries, end = [], []
+        for i in list(live):
+            p = live[i].pop(0)
+            entries.append({"id": i, "tokens": p, "want": list(range(len(p)))})
+            if not live[i]:
+                end.append(i)
+                del live[i]
+        out = rp.step(entries, end)
+        off = 0
+        for e in entries:
+            got[e["id"]].append(out[off:off + len(e["tokens"])])
+            off += len(e["tokens"])
+    for i, toks in reqs.items():
+        close(torch.cat(got[i], 0), O.forward(cfg, Wr, toks), dtype, f"{i} on reused pages")
+    assert eng.kv.num_free() == 6 and eng.state_pool.num_free() == 2
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_long_decode(mode):
+    """A short prompt, then 150 tokens one by one: state and cache carry on."""
+    device, dtype = mode
+    _skip_if_wrong_device(device)
+    cfg = make_cfg("RmA-LmR-", loop=(0, 2, 2))
+    W = O.random_weights(cfg, seed=8)
+    eng = build_engine(cfg, W, dtype)
+    toks = tokens_for(cfg, 170, 9)
+    want = O.forward(cfg, rounded(W, dtype), toks)
+    parts = [toks[:20]] + [[t] for t in toks[20:]]
+    got = replay(eng, [[("a", p, k == len(parts) - 1)] for k, p in enumerate(parts)])["a"]
+    close(got, want, dtype, "long decode")
+
+
+VARIANTS = {
+    # values that are often equal or 1, made different or extreme
+    "one-head": dict(heads=1, kv_heads=1, lat_heads=1, ret_heads=1, decay=[0.9]),
+    "heads-equal-kv-heads": dict(heads=3, kv_heads=3),
+    "partly-rotated": dict(rot_dim=10, rot_dims=4, ret_rot_dims=6),
+    "unrotated": dict(rot_dims=0, ret_rot_dims=0),
+    "top-1": dict(top=1, experts=5),
+    "all-experts": dict(top=4, experts=4),
+    "no-shared-expert": dict(shared_ff=0),
+    "unit-constants": dict(embed_scale=1.0, logit_scale=1.0, scale=1.0, diff=0.0, softcap=None),
+    "one-stream": dict(streams=1),
+    "plain-residual": dict(streams=None),
+    "five-streams": dict(streams=5),
+    "no-loop": dict(loop=None),
+    "loop-thrice-to-the-end": dict(loop=(2, 5, 3)),
+    "wide-values": dict(vdim=44, ret_vdim=68, ret_dim=8, ret_rot_dims=8, lat_vdim=36),
+    "big-latent": dict(kv_rank=72, rot_dim=24, lat_dim=4, q_rank=7),
+}
+
+
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("variant", sorted(VARIANTS))
+def test_other_sizes(mode, variant):
+    device, dtype = mode
+    _skip_if_wrong_device(device)
+    cfg = make_cfg("AmLmR-Rm", **VARIANTS[variant]) if variant != "loop-thrice-to-the-end" else \
+        make_cfg("AmLmR-RmL-", **VARIANTS[variant])
+    W = O.random_weights(cfg, seed=11)
+    eng = build_engine(cfg, W, dtype)
+    toks = tokens_for(cfg, 40, 12)
+    want = O.forward(cfg, rounded(W, dtype), toks)
+    parts = cut(toks, [13, 2, 1, 1, 9])
+    got = replay(eng, [[("a", p, k == len(parts) - 1)] for k, p in enumerate(parts)])["a"]
+    close(got, want, dtype, variant)
+
+
+def test_config_reader_takes_every_constant():
+    """Every size and constant of config.json lands in the spec."""
+    cfg = make_cfg()
+    spec = suzulix_spec_from_dict(cfg)
+    assert (spec.layer_style, spec.streams, spec.hyper, spec.loop) == ("hyper", 3, True, (1, 3, 2))
+    assert (spec.embed_scale, spec.logit_scale, spec.norm_eps, spec.tied_head) == (3.0, 0.4, 1e-5, True)
+    assert spec.layer_runs() == [0, 1, 2, 1, 2, 3, 4]
+    la, da, rt = (spec.layers[i].mixer for i in range(3))
+    assert (la.kind, la.heads, la.dim, la.vdim, la.kv_rank, la.q_rank, la.rot_dim, la.rot_dims,
+            la.rot_base, la.scale, la.rot_layout, la.sink, la.gate) == (
+        "latent_attention", 3, 8, 14, 18, 22, 6, 6, 50.0, 0.23, "half", False, "channel")
+    assert (da.kind, da.heads, da.kv_heads, da.dim, da.vdim, da.rot_dims, da.rot_base, da.scale,
+            da.softcap, da.diff, da.rot_layout) == (
+        "diff_attention", 6, 2, 12, 10, 8, 50.0, 0.23, 4.0, 0.3, "interleaved")
+    assert (rt.kind, rt.heads, rt.dim, rt.vdim, rt.rot_dims, rt.decay, rt.rot_layout) == (
+        "retention", 2, 20, 12, 12, [0.7, 0.995], "half")
+    assert la.has_kv and da.has_kv and rt.has_state and not rt.has_kv and not da.has_state
+    r = spec.layers[0].router
+    assert (r.experts, r.top, r.ff, r.shared_ff, r.act, r.gated, r.bias, r.shared_gate, r.score,
+            r.renorm, r.groups) == (12, 3, 20, 28, "relu2", False, True, True, "softmax", True, 1)
+    assert spec.layers[3].mlp_kind is None
+    plain = suzulix_spec_from_dict(make_cfg(streams=None, loop=None))
+    assert (plain.streams, plain.hyper, plain.loop) == (1, False, None)
+    for bad_loop in ({"start": 3, "stop": 2, "times": 2}, {"start": 0, "stop": 9, "times": 2},
+                     {"start": 0, "stop": 2, "times": 0}):
+        bad = copy.deepcopy(cfg)
+        bad["loop"] = bad_loop
+        with pytest.raises(ValueError):
+            suzulix_spec_from_dict(bad)
+    bad = copy.deepcopy(cfg)
+    bad["layers"][0]["type"] = "convolution"
+    with pytest.raises(ValueError):
+        suzulix_spec_from_dict(bad)
+
+
+def test_every_pass_has_its_own_cache_and_state():
+    """Pages and state slots are kept per layer RUN: a looped layer has one
+    set per pass. The latent layer caches kv_rank + rot_dim channels with the
+    values a view of them; differential attention caches two key maps per
+    value head; retention keeps no pages."""
+    cfg = make_cfg()
+    eng = build_engine(cfg, O.random_weights(cfg), "fp32", blocks=8)
+    if eng.device == "cuda":
+        pytest.skip("covered on CPU runs")
+    assert len(eng.kv.layers) == 7 and len(eng.state_pool.tensors) == 7
+    k, v = eng.kv.layers[0]
+    assert k.shape[2:] == (1, 24) and v.shape[2:] == (1, 18) and v.data_ptr() == k.data_ptr()
+    for run in (1, 3, 6):
+        k, v = eng.kv.layers[run]
+        assert k.shape[2:] == (4, 12) and v.shape[2:] == (2, 10)
+    assert eng.kv.layers[1][0].data_ptr() != eng.kv.layers[3][0].data_ptr()
+    for run in (2, 4, 5):
+        assert eng.kv.layers[run] == (None, None)
+        assert eng.state_pool.tensors[run]["S"].shape[1:] == (2, 12, 20)
+    assert eng.state_pool.tensors[2]["S"].data_ptr() != eng.state_pool.tensors[4]["S"].data_ptr()
+    assert eng.model.lm_head is eng.model.embed
+
+
+def test_checkpoint_folder_roundtrip(tmp_path):
+    """A folder with config.json and model.safetensors (bfloat16) is found by
+    its architecture name and serves the oracle's logits."""
+    from safetensors.torch import save_file
+
+    cfg = make_cfg("RmAmL-", width=32, experts=4, top=2, expert_ff=8, shared_ff=8, loop=(0, 2, 3),
+                   streams=2)
+    W = {k: v.to(torch.bfloat16) for k, v in O.random_weights(cfg, seed=2).items()}
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    save_file({k: v.contiguous() for k, v in W.items()}, str(tmp_path / "model.safetensors"))
+    if torch.cuda.is_available():
+        pytest.skip("covered on CPU runs")
+    eng = LLMEngine({"model": str(tmp_path), "dtype": "fp32", "kv_num_blocks": 16, "kv_block_size": 8,
+                     "max_batch_size": 2, "state_slots": 2, "tokenizer_check": False})
+    assert eng.spec.architecture == "Suzulix" and eng.model.runs == [0, 1, 0, 1, 0, 1, 2]
+    toks = tokens_for(cfg, 20, 1)
+    got = replay(eng, [[("a", toks, True)]])["a"]
+    close(got, O.forward(cfg, {k: v.float() for k, v in W.items()}, toks), "fp32", "folder")
+
+
+# --------------------------------------------------------------------------
+# generation through the engine's own entry point and scheduler
+
+
+@pytest.mark.parametrize("mode", MODES[:2])
+def test_greedy_generation_matches_oracle(mode, model_case):
+    device, dtype = mode
+    _skip_if_wrong_device(device)
+    cfg, W = model_case
+    eng = build_engine(cfg, W, dtype, max_prefill_chunk=16)     # prompt read in portions
+    prompt = tokens_for(cfg, 37, 30)
+    out, reason = eng.generate(prompt, SamplingParams(max_new_tokens=24, stop_on_eos=False))
+    assert reason == "length"
+    assert out == O.greedy(cfg, W, prompt, 24)
+
+
+@pytest.mark.parametrize("mode", MODES)
+def test_scheduler_batches_equal_solo(mode, model_case):
+    """Five requests through add_request/step with two slots: admission waits
+    for a free slot, portions and decodes share forwards, and every output
+    equals the request generated alone."""
+    device, dtype = mode
+    _skip_if_wrong_device(device)
+    cfg, W = model_case
+    prompts = [tokens_for(cfg, n, 40 + n) for n in (5, 33, 1, 18, 9)]
+    params = SamplingParams(max_new_tokens=10, stop_on_eos=False)
+    solo = []
+    eng = build_engine(cfg, W, dtype, max_prefill_chunk=12)
+    for p in prompts:
+        solo.append(eng.generate(p, params)[0])
+    eng2 = build_engine(cfg, W, dtype, slots=2, max_prefill_chunk=12)
+    rids = [eng2.add_request(p, params) for p in prompts]
+    for _ in range(400):
+        if all(eng2.requests[r].finished for r in rids):
+            break
+        eng2.step()
+    if dtype == "fp32":
+        assert [eng2.requests[r].output_ids for r in rids] == solo
+    else:
+        assert all(len(eng2.requests[r].output_ids) == 10 for r in rids)
+    assert eng2.state_pool.num_free() == 2 and eng2.kv.num_free() == eng2.kv.num_blocks
+
+
+@gpu
+@pytest.mark.parametrize("dtype", ["fp32", "bf16"])
+def test_decode_graph_equals_eager(dtype, model_case):
+    """Decode-only steps replay a captured graph per batch bucket; several
+    replays, with eager portions between them, equal the eager engine."""
+    cfg, W = model_case
+    reqs = {"a": tokens_for(cfg, 40, 50), "b": tokens_for(cfg, 33, 51), "c": tokens_for(cfg, 21, 52)}
+    sched = [[("a", reqs["a"][:20], False), ("b", reqs["b"][:9], False)]]
+    for k in range(12):
+        sched.append([("a", [reqs["a"][20 + k]], False), ("b", [reqs["b"][9 + k]], False)])
+    sched.append([("c", reqs["c"][:15], False), ("a", [reqs["a"][32]], False)])
+    for k in range(6):
+        sched.append([("a", [reqs["a"][33 + k]], False), ("b", [reqs["b"][21 + k]], False),
+                      ("c", [reqs["c"][15 + k]], False)])
+    outs = []
+    for graph in (False, True):
+        eng = build_engine(cfg, W, dtype, use_hipgraph=graph)
+        outs.append(replay(eng, copy.deepcopy(sched)))
+        if graph:
+            assert any(e["graph"] is not None for e in eng._graphs.values())
+    for i in reqs:
+        assert torch.equal(outs[0][i], outs[1][i]), f"graph replay differs for {i}"
+
+
+def test_named_sizes_build():
+    """The registry's Suzulix sizes parse; the CPU-test size serves tokens."""
+    from opsagent_amd.engine.config import get_model_spec
+
+    for name in ("suzulix-tiny", "suzulix-micro", "suzulix-4l2k", "suzulix-4l4k"):
+        spec = get_model_spec(name)
+        assert spec.architecture == "Suzulix" and spec.layer_style == "hyper"
+    if torch.cuda.is_available():
+        pytest.skip("generation on the CPU path is covered on CPU runs")
+    eng = LLMEngine({"model": "suzulix-tiny", "dtype": "fp32", "kv_num_blocks": 32,
+                     "kv_block_size": 8, "max_batch_size": 2, "state_slots": 2,
+                     "tokenizer_check": False})
+    out, reason = eng.generate([5, 6, 7, 8, 9], SamplingParams(max_new_tokens=6, stop_on_eos=False))
+    assert len(out) == 6 and reason == "length"
