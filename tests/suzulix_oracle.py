@@ -14,6 +14,34 @@ import torch
 F64 = torch.float64
 
 
+# Where the product path may hold bfloat16 (projection outputs, normed sublayer
+# inputs, mixer outputs before the output projection) the oracle can round too:
+# the difference to the unrounded run shows how far rounding alone moves a
+# position. Off by default.
+_ROUND = [None]
+
+
+class rounding:
+    """with rounding(fn): every low-precision point applies fn."""
+
+    def __init__(self, fn):
+        self.fn = fn
+
+    def __enter__(self):
+        _ROUND[0] = self.fn
+
+    def __exit__(self, *a):
+        _ROUND[0] = None
+
+
+def lowp(x):
+    return x if _ROUND[0] is None else _ROUND[0](x)
+
+
+def proj(x, w):
+    return lowp(x @ w.T)
+
+
 def layer_norm(x, w, b, eps):
     mu = x.mean(-1, keepdim=True)
     var = ((x - mu) ** 2).mean(-1, keepdim=True)
@@ -57,20 +85,20 @@ def latent_attention(h, W, p, m, eps):
     H, D, rot, Dv, R = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
     rd, rb = m["rot"]["dims"], m["rot"]["base"]
     pos = torch.arange(T)
-    cq = unit_rms(h @ W[p + "dq"].T, eps) * W[p + "dq.norm"]
-    q = (cq @ W[p + "uq"].T).reshape(T, H, D + rot)
-    d = h @ W[p + "dkv"].T
+    cq = lowp(unit_rms(proj(h, W[p + "dq"]), eps) * W[p + "dq.norm"])
+    q = proj(cq, W[p + "uq"]).reshape(T, H, D + rot)
+    d = proj(h, W[p + "dkv"])
     c = unit_rms(d[:, :R], eps) * W[p + "dkv.norm"]
     kr = turn(d[:, R:R + rot], pos, rd, rb, "half")
-    ku = (c @ W[p + "uk"].T).reshape(T, H, D)
-    v = (c @ W[p + "uv"].T).reshape(T, H, Dv)
+    ku = proj(c, W[p + "uk"]).reshape(T, H, D)
+    v = proj(c, W[p + "uv"]).reshape(T, H, Dv)
     out = torch.zeros(T, H, Dv, dtype=F64)
     for hh in range(H):
         qr = turn(q[:, hh, D:], pos, rd, rb, "half")
         s = (q[:, hh, :D] @ ku[:, hh].T + qr @ kr.T) * m["scale"]
         out[:, hh] = softmax_rows(s) @ v[:, hh]
-    out = out.reshape(T, H * Dv) * sigmoid(h @ W[p + "g"].T)
-    return out @ W[p + "o"].T
+    out = lowp(out.reshape(T, H * Dv) * sigmoid(proj(h, W[p + "g"])))
+    return proj(out, W[p + "o"])
 
 
 def diff_lambda(W, p, m):
@@ -83,9 +111,9 @@ def diff_attention(h, W, p, m, eps):
     H, G, D, Dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
     rot = m.get("rot") or {"dims": 0, "base": 1.0}
     pos = torch.arange(T)
-    q = (h @ W[p + "q"].T).reshape(T, H, 2, D)
-    k = (h @ W[p + "k"].T).reshape(T, G, 2, D)
-    v = (h @ W[p + "v"].T).reshape(T, G, Dv)
+    q = proj(h, W[p + "q"]).reshape(T, H, 2, D)
+    k = proj(h, W[p + "k"]).reshape(T, G, 2, D)
+    v = proj(h, W[p + "v"]).reshape(T, G, Dv)
     lam = diff_lambda(W, p, m)
     cap = m.get("softcap")
     out = torch.zeros(T, H, Dv, dtype=F64)
@@ -101,8 +129,8 @@ def diff_attention(h, W, p, m, eps):
             maps.append(softmax_rows(s) @ v[:, g])
         o = maps[0] - lam * maps[1]
         out[:, hh] = unit_rms(o, eps) * (1.0 - m["diff"])
-    out = out.reshape(T, H * Dv) * sigmoid(h @ W[p + "g"].T)
-    return out @ W[p + "o"].T
+    out = lowp(out.reshape(T, H * Dv) * sigmoid(proj(h, W[p + "g"])))
+    return proj(out, W[p + "o"])
 
 
 def retention(h, W, p, m, eps):
@@ -110,9 +138,9 @@ def retention(h, W, p, m, eps):
     H, D, Dv = m["heads"], m["dim"], m["vdim"]
     rot = m.get("rot") or {"dims": 0, "base": 1.0}
     pos = torch.arange(T)
-    q = (h @ W[p + "q"].T).reshape(T, H, D)
-    k = (h @ W[p + "k"].T).reshape(T, H, D)
-    v = (h @ W[p + "v"].T).reshape(T, H, Dv)
+    q = proj(h, W[p + "q"]).reshape(T, H, D)
+    k = proj(h, W[p + "k"]).reshape(T, H, D)
+    v = proj(h, W[p + "v"]).reshape(T, H, Dv)
     out = torch.zeros(T, H, Dv, dtype=F64)
     for hh in range(H):
         qq = turn(q[:, hh], pos, rot["dims"], rot["base"], "half")
@@ -121,13 +149,13 @@ def retention(h, W, p, m, eps):
         for t in range(T):
             S = float(m["decay"][hh]) * S + torch.outer(kk[t], v[t, hh])
             out[t, hh] = S.T @ qq[t]
-    z = h @ W[p + "g"].T
-    y = unit_rms(out, eps).reshape(T, H * Dv) * (z * sigmoid(z))
-    return y @ W[p + "o"].T
+    z = proj(h, W[p + "g"])
+    y = lowp(unit_rms(out, eps).reshape(T, H * Dv) * (z * sigmoid(z)))
+    return proj(y, W[p + "o"])
 
 
 def expert(h, W, p):
-    return torch.clamp(h @ W[p + "up"].T, min=0.0) ** 2 @ W[p + "down"].T
+    return proj(lowp(torch.clamp(proj(h, W[p + "up"]), min=0.0) ** 2), W[p + "down"])
 
 
 def moe_ff(h, W, p, mlp):
@@ -180,12 +208,12 @@ def forward(cfg, W, tokens, layers_out=None):
             else:
                 rd, wr, mix = torch.ones(1, dtype=F64), torch.ones(1, dtype=F64), torch.ones(1, 1, dtype=F64)
             u = sum(rd[s] * xs[s] for s in range(S))
-            y = fn(layer_norm(u, W[f"{p}norm{q}"], W[f"{p}norm{q}.b"], eps))
+            y = fn(lowp(layer_norm(u, W[f"{p}norm{q}"], W[f"{p}norm{q}.b"], eps)))
             xs = [sum(mix[s, t] * xs[s] for s in range(S)) + wr[t] * y for t in range(S)]
         if layers_out is not None:
             layers_out.append(sum(xs))
     x = sum(xs)
-    return (layer_norm(x, W["final.norm"], W["final.norm.b"], eps) @ W["embed"].T
+    return (proj(lowp(layer_norm(x, W["final.norm"], W["final.norm.b"], eps)), W["embed"])
             * cfg.get("logit_scale", 1.0))
 
 

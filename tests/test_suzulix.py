@@ -49,6 +49,60 @@ def close(got, want, dtype, what="", loose=1.0):
         assert err < 3e-2 * loose and worst < 1.5e-1 * loose, f"{what}: rel rms {err:.3e}, worst {worst:.3e}"
 
 
+def _bf16_nearest(x):
+    return x.to(torch.bfloat16).double()
+
+
+def _bf16_chop(x):
+    """Rounding toward zero: another realisation of the same noise level."""
+    f = x.float()
+    return (f.view(torch.int32) & -65536).view(torch.float32).double()
+
+
+def oracle_runs(cfg, W, toks, dtype, layers=False):
+    """The oracle's logits (and, with `layers`, the sum of the streams after
+    every layer run), and in bf16 mode the same from runs whose low-precision
+    points are rounded to bfloat16 in two ways: how far rounding alone moves
+    each position."""
+    exact_layers = []
+    exact = O.forward(cfg, W, toks, exact_layers)
+    noisy = []
+    if dtype == "bf16":
+        for fn in (_bf16_nearest, _bf16_chop):
+            with O.rounding(fn):
+                ls = []
+                lg = O.forward(cfg, W, toks, ls)
+            noisy.append((lg, ls))
+    return exact, exact_layers, noisy
+
+
+def close_rows(got, want, noisy, dtype, what=""):
+    """Row by row (a row is a position). float32: the strict bounds of close().
+    bfloat16: a row may be as far from the oracle as 3e-2 of its size plus four
+    times what rounding alone moved it in the oracle's own rounded runs — a
+    position whose value hangs on a near-zero quantity (the sign of a single
+    key.query product behind a unit norm, say) is allowed what its
+    conditioning allows, and every other row the plain bound. Of 20 rows or
+    more, one in 30 (at least one) may still be further off: a router's close
+    call that flips in the engine's rounding and in neither of the oracle's."""
+    if dtype == "fp32":
+        return close(got, want, dtype, what)
+    got, want = got.detach().double().cpu(), want.detach().double().cpu()
+    assert got.shape == want.shape, (got.shape, want.shape)
+    size = want.pow(2).mean(-1).sqrt() + 1e-9
+    err = (got - want).pow(2).mean(-1).sqrt() / size
+    moved = torch.stack([(n.double() - want).pow(2).mean(-1).sqrt() / size for n in noisy]).max(0).values
+    bad = (err > 3e-2 + 4.0 * moved).nonzero().flatten().tolist()
+    allowed = max(1, err.numel() // 30) if err.numel() >= 20 else 0
+    assert len(bad) <= allowed, f"{what}: rows {bad[:8]}: err {err[bad[:8]].tolist()}, rounding alone {moved[bad[:8]].tolist()}"
+
+
+def model_close(got, cfg, W, toks, dtype, what=""):
+    """Logits of every position of `toks` against the oracle."""
+    exact, _, noisy = oracle_runs(cfg, rounded(cfg, W, dtype), toks, dtype)
+    close_rows(got, exact, [lg for lg, _ in noisy], dtype, what)
+
+
 def make_cfg(pattern="LmAmRmR-Am", width=40, vocab=97, **kw):
     base = dict(heads=6, kv_heads=2, dim=12, vdim=10, kv_rank=18, q_rank=22, rot_dim=6,
                 lat_heads=3, lat_dim=8, lat_vdim=14, rot_dims=8, rot_base=50.0, scale=0.23,
@@ -67,11 +121,22 @@ def x16_cfg(pattern="LmAmRmR-Am"):
                     expert_ff=32, shared_ff=48, streams=2)
 
 
-def rounded(W, dtype):
-    """The oracle sees the weights the engine holds (bfloat16-rounded in bf16 mode)."""
-    if dtype == "bf16":
-        return {k: v.to(torch.bfloat16).float() for k, v in W.items()}
-    return W
+def rounded(cfg, W, dtype):
+    """The oracle sees the weights the engine holds. In bf16 mode they are
+    bfloat16-rounded, and every router is made decisive first: the `top`
+    largest biases are raised by 4, so that rounding noise in a router's input
+    does not flip an expert at a close call (which would move single tokens
+    by far more than rounding does). Which experts a token gets still depends
+    on the token; float32 runs keep the undoctored routers."""
+    if dtype != "bf16":
+        return W
+    W = dict(W)
+    for i, layer in enumerate(cfg["layers"]):
+        if layer.get("mlp") is not None:
+            b = W[f"l{i}.mlp.router.b"].clone()
+            b[b.topk(layer["mlp"]["router"]["top"]).indices] += 4.0
+            W[f"l{i}.mlp.router.b"] = b
+    return {k: v.to(torch.bfloat16).float() for k, v in W.items()}
 
 
 def build_engine(cfg, W, dtype="fp32", blocks=64, block_size=8, slots=4, **extra):
@@ -80,7 +145,7 @@ def build_engine(cfg, W, dtype="fp32", blocks=64, block_size=8, slots=4, **extra
         "kv_block_size": block_size, "max_batch_size": slots, "state_slots": slots,
         "tokenizer_check": False, "max_seq_len": 4096, "max_prefill_chunk": 4096,
     }, **extra))
-    eng.model.load_named_tensors(rounded(W, dtype))
+    eng.model.load_named_tensors(rounded(cfg, W, dtype))
     return eng
 
 
@@ -358,12 +423,11 @@ def test_mixer_alone(mode, kind, k):
     W = O.random_weights(cfg, seed=3 + k)
     eng = build_engine(cfg, W, dtype)
     toks = tokens_for(cfg, 29, k)
-    layers = []
-    O.forward(cfg, rounded(W, dtype), toks, layers)
+    _, layers, noisy = oracle_runs(cfg, rounded(cfg, W, dtype), toks, dtype)
     eng.model.trace_layers = []
     replay(eng, [[("a", toks[:17], False)], [("a", toks[17:], True)]])
     got = torch.cat(eng.model.trace_layers, 0)
-    close(got, layers[0], dtype, f"{kind} geometry {k}")
+    close_rows(got, layers[0], [ls[0] for _, ls in noisy], dtype, f"{kind} geometry {k}")
 
 
 @pytest.mark.parametrize("mode", MODES)
@@ -378,7 +442,7 @@ def test_slow_decay_remembers_the_first_token(mode):
     eng = build_engine(cfg, W, dtype)
     toks = tokens_for(cfg, 400, 6)
     other = [(toks[0] + 1) % cfg["vocab"]] + toks[1:]
-    Wr = rounded(W, dtype)
+    Wr = rounded(cfg, W, dtype)
     want = O.forward(cfg, Wr, toks)[-3:]
     assert (want - O.forward(cfg, Wr, other)[-3:]).abs().max() > 1e-3
     parts = [toks[:200], toks[200:397]] + [[t] for t in toks[397:]]
@@ -402,7 +466,7 @@ def test_ungated_experts_paths(mode, sizes):
     mlp = eng.model.layers[1].mlp
     g = torch.Generator().manual_seed(1)
     x = torch.randn(37, C, generator=g).to(tdtype(dtype))
-    Wd = {k: v.double() for k, v in rounded(W, dtype).items()}
+    Wd = {k: v.double() for k, v in rounded(cfg, W, dtype).items()}
     want = O.moe_ff(x.double(), Wd, "l1.mlp.", cfg["layers"][1]["mlp"])
     for path in ("pairs", "sorted"):
         mlp.force_path = path
@@ -445,14 +509,13 @@ def test_layers_and_logits_whole_prompt(mode, model_case):
     cfg, W = model_case
     eng = build_engine(cfg, W, dtype)
     toks = tokens_for(cfg, 45, 2)
-    layers = []
-    want = O.forward(cfg, rounded(W, dtype), toks, layers)
+    want, layers, noisy = oracle_runs(cfg, rounded(cfg, W, dtype), toks, dtype)
     eng.model.trace_layers = []
     got = replay(eng, [[("a", toks, True)]])["a"]
     assert len(eng.model.trace_layers) == len(layers) == 7      # two looped layers count twice
     for i, x in enumerate(eng.model.trace_layers):
-        close(x, layers[i], dtype, f"sum of streams after run {i}")
-    close(got, want, dtype, "logits")
+        close_rows(x, layers[i], [ls[i] for _, ls in noisy], dtype, f"sum of streams after run {i}")
+    close_rows(got, want, [lg for lg, _ in noisy], dtype, "logits")
 
 
 @pytest.mark.parametrize("mode", MODES)
@@ -461,13 +524,11 @@ def test_first_tokens(mode, model_case):
     _skip_if_wrong_device(device)
     cfg, W = model_case
     eng = build_engine(cfg, W, dtype)
-    Wr = rounded(W, dtype)
     for n in (1, 2, 3):
         toks = tokens_for(cfg, n, 10 + n)
-        want = O.forward(cfg, Wr, toks)
-        close(replay(eng, [[("s", toks, True)]])["s"], want, dtype, f"{n} tokens at once")
-        close(replay(eng, [[("s", [t], k == n - 1)] for k, t in enumerate(toks)])["s"], want, dtype,
-              f"{n} tokens one by one")
+        model_close(replay(eng, [[("s", toks, True)]])["s"], cfg, W, toks, dtype, f"{n} tokens at once")
+        model_close(replay(eng, [[("s", [t], k == n - 1)] for k, t in enumerate(toks)])["s"], cfg, W,
+                    toks, dtype, f"{n} tokens one by one")
 
 
 @pytest.mark.parametrize("mode", MODES)
@@ -480,10 +541,9 @@ def test_portions_and_decode(mode, model_case, sizes):
     cfg, W = model_case
     eng = build_engine(cfg, W, dtype)
     toks = tokens_for(cfg, 61, 3)
-    want = O.forward(cfg, rounded(W, dtype), toks)
     parts = cut(toks, sizes)
     got = replay(eng, [[("a", p, k == len(parts) - 1)] for k, p in enumerate(parts)])["a"]
-    close(got, want, dtype, f"portions {sizes}")
+    model_close(got, cfg, W, toks, dtype, f"portions {sizes}")
     assert eng.kv.num_free() == eng.kv.num_blocks and eng.state_pool.num_free() == 4
 
 
@@ -495,7 +555,6 @@ def test_unequal_batch_equals_alone(mode, model_case):
     _skip_if_wrong_device(device)
     cfg, W = model_case
     eng = build_engine(cfg, W, dtype)
-    Wr = rounded(W, dtype)
     reqs = {"a": tokens_for(cfg, 53, 4), "b": tokens_for(cfg, 9, 5), "c": tokens_for(cfg, 1, 7),
             "d": tokens_for(cfg, 30, 7)}
     plan = {"a": cut(reqs["a"], [11, 2, 1, 1, 19]), "b": cut(reqs["b"], [1]),
@@ -511,7 +570,7 @@ def test_unequal_batch_equals_alone(mode, model_case):
         k += 1
     got = replay(eng, schedule)
     for i, toks in reqs.items():
-        close(got[i], O.forward(cfg, Wr, toks), dtype, f"request {i} in a mixed batch")
+        model_close(got[i], cfg, W, toks, dtype, f"request {i} in a mixed batch")
 
 
 @pytest.mark.parametrize("mode", MODES)
@@ -523,7 +582,6 @@ def test_pages_and_slots_used_again(mode, model_case):
     _skip_if_wrong_device(device)
     cfg, W = model_case
     eng = build_engine(cfg, W, dtype, blocks=6, block_size=8, slots=2)
-    Wr = rounded(W, dtype)
     lens = [20, 17, 25, 3, 24, 9, 22]
     reqs = {"r%d" % k: tokens_for(cfg, n, 20 + k) for k, n in enumerate(lens)}
     rp = TraceReplayer(eng)
@@ -549,7 +607,7 @@ def test_pages_and_slots_used_again(mode, model_case):
             got[e["id"]].append(out[off:off + len(e["tokens"])])
             off += len(e["tokens"])
     for i, toks in reqs.items():
-        close(torch.cat(got[i], 0), O.forward(cfg, Wr, toks), dtype, f"{i} on reused pages")
+        model_close(torch.cat(got[i], 0), cfg, W, toks, dtype, f"{i} on reused pages")
     assert eng.kv.num_free() == 6 and eng.state_pool.num_free() == 2
 
 
@@ -562,10 +620,9 @@ def test_long_decode(mode):
     W = O.random_weights(cfg, seed=8)
     eng = build_engine(cfg, W, dtype)
     toks = tokens_for(cfg, 170, 9)
-    want = O.forward(cfg, rounded(W, dtype), toks)
     parts = [toks[:20]] + [[t] for t in toks[20:]]
     got = replay(eng, [[("a", p, k == len(parts) - 1)] for k, p in enumerate(parts)])["a"]
-    close(got, want, dtype, "long decode")
+    model_close(got, cfg, W, toks, dtype, "long decode")
 
 
 VARIANTS = {
@@ -598,10 +655,9 @@ def test_other_sizes(mode, variant):
     W = O.random_weights(cfg, seed=11)
     eng = build_engine(cfg, W, dtype)
     toks = tokens_for(cfg, 40, 12)
-    want = O.forward(cfg, rounded(W, dtype), toks)
     parts = cut(toks, [13, 2, 1, 1, 9])
     got = replay(eng, [[("a", p, k == len(parts) - 1)] for k, p in enumerate(parts)])["a"]
-    close(got, want, dtype, variant)
+    model_close(got, cfg, W, toks, dtype, variant)
 
 
 def test_config_reader_takes_every_constant():
