@@ -274,10 +274,9 @@ class RoutedExperts(nn.Module):
 
         T, C = x.shape
         I, top = self.r.ff, self.r.top
-        if not self.gated:
-            return mx.moe_pairs_plain(x.contiguous(), self.w13, self.w2, idx, wts, self.act)
-        fast_act = self.act == "silu" or (isinstance(self.act, tuple)
-                                          and self.act[0] == "clamp_swish")
+        fast_act = (self.act == "silu" or (isinstance(self.act, tuple)
+                                           and self.act[0] == "clamp_swish")
+                    or (not self.gated and self.act == "relu2"))
         if (x.is_cuda and x.dtype == torch.bfloat16 and fast_act
                 and C % 16 == 0 and I % 16 == 0 and self.force_path is None):
             # the framework's grouped expert GEMV kernels (pair- or expert-major)
@@ -287,6 +286,8 @@ class RoutedExperts(nn.Module):
                                     wts.reshape(-1).contiguous(), I, False,
                                     num_experts=self.r.experts, act=self.act)
             return y.view(T, top, C).float().sum(1).to(x.dtype)
+        if not self.gated:
+            return mx.moe_pairs_plain(x.contiguous(), self.w13, self.w2, idx, wts, self.act)
         return mx.moe_pairs_mlp(x.contiguous(), self.w13, self.w2, idx, wts, self.act)
 
     def _sorted(self, x, idx, wts):

@@ -359,11 +359,16 @@ def moe_grouped_mlp(
         block column per EXPERT; weights stream once per GROUP of 8 matched
         pairs, cutting the weight traffic up to 8x at big decode batches
     act: None / "silu", or ("clamp_swish", limit, alpha) for the clamped gate
-    g' = min(g, limit), u' = clamp(u, -limit, limit), g' sigmoid(alpha g') (u' + 1).
+    g' = min(g, limit), u' = clamp(u, -limit, limit), g' sigmoid(alpha g') (u' + 1),
+    or "relu2" for UNGATED experts: w13 is [E, I, K] (up rows alone) and the
+    middle activation is relu(up x)^2.
     """
     if isinstance(act, tuple):
         assert act[0] == "clamp_swish"
         actk, limit, alpha = 2, float(act[1]), float(act[2])
+    elif act == "relu2":
+        assert w13.shape[1] == i_local
+        actk, limit, alpha = 3, 0.0, 0.0
     else:
         assert act in (None, "silu")
         actk, limit, alpha = 0, 0.0, 0.0

@@ -41,23 +41,25 @@ __device__ __forceinline__ void hc_st4(bf16s* p, int64_t i, const float* v) {
 // The sums over streams run in stream order, so a token's result is the same
 // in every batch. The first 256 * HC_NR channels of u stay in registers
 // between the passes; wider rows rebuild u from the (just written) streams.
-template <typename TC, bool VEC>
+template <typename TC, bool VEC, int NSTR>
 __global__ __launch_bounds__(256) void hyper_norm_kernel(
-    float* __restrict__ streams, int S, const TC* __restrict__ y, int64_t ys,
+    float* __restrict__ streams, int S_rt, const TC* __restrict__ y, int64_t ys,
     const TC* __restrict__ y2, int64_t y2s, const float* __restrict__ g2, int64_t g2s,
     const float* __restrict__ mix, const float* __restrict__ write,
     const float* __restrict__ read, const float* __restrict__ w, const float* __restrict__ b,
     TC* __restrict__ out, int C, float eps) {
     __shared__ float red_a[16], red_b[16];
-    __shared__ float smix[HC_MAXS * HC_MAXS], swr[HC_MAXS], srd[HC_MAXS];
+    __shared__ float smix[NSTR * NSTR], swr[NSTR], srd[NSTR];
     constexpr int W = VEC ? 4 : 1;
     constexpr int NS = HC_NR / W;
+    // NSTR < HC_MAXS: exactly NSTR streams (loops fold); NSTR == HC_MAXS: any count up to it
+    const int S = NSTR == HC_MAXS ? S_rt : NSTR;
     const int t = blockIdx.x, tid = threadIdx.x;
-    if (tid < HC_MAXS * HC_MAXS) {
-        const int s = tid / HC_MAXS, k = tid % HC_MAXS;
+    if (tid < NSTR * NSTR) {
+        const int s = tid / NSTR, k = tid % NSTR;
         smix[tid] = (mix && s < S && k < S) ? mix[s * S + k] : 0.0f;
     }
-    if (tid < HC_MAXS) {
+    if (tid < NSTR) {
         swr[tid] = (write && tid < S) ? write[tid] : 0.0f;
         srd[tid] = (read && tid < S) ? read[tid] : 0.0f;
     }
@@ -68,9 +70,9 @@ __global__ __launch_bounds__(256) void hyper_norm_kernel(
     const float gate = (y2 && g2) ? sigmoidf_(g2[(int64_t)t * g2s]) : 1.0f;
     // channels c .. c+W-1: update the streams, return u
     auto step = [&](int c, float* u) {
-        float x[HC_MAXS][W];
+        float x[NSTR][W];
 #pragma unroll
-        for (int s = 0; s < HC_MAXS; ++s) {
+        for (int s = 0; s < NSTR; ++s) {
             if (s < S) {
                 if (VEC) hc_ld4(xs + (int64_t)s * C, c, x[s]);
                 else x[s][0] = xs[(int64_t)s * C + c];
@@ -86,16 +88,16 @@ __global__ __launch_bounds__(256) void hyper_norm_kernel(
 #pragma unroll
                 for (int e = 0; e < W; ++e) yy[e] += gate * a[e];
             }
-            float nx[HC_MAXS][W];
+            float nx[NSTR][W];
 #pragma unroll
-            for (int k = 0; k < HC_MAXS; ++k) {
+            for (int k = 0; k < NSTR; ++k) {
                 if (k < S) {
 #pragma unroll
                     for (int e = 0; e < W; ++e) {
                         float acc = 0.0f;
 #pragma unroll
-                        for (int s = 0; s < HC_MAXS; ++s)
-                            if (s < S) acc = fmaf(smix[s * HC_MAXS + k], x[s][e], acc);
+                        for (int s = 0; s < NSTR; ++s)
+                            if (s < S) acc = fmaf(smix[s * NSTR + k], x[s][e], acc);
                         nx[k][e] = fmaf(swr[k], yy[e], acc);
                     }
                     if (VEC) hc_st4(xs + (int64_t)k * C, c, nx[k]);
@@ -103,7 +105,7 @@ __global__ __launch_bounds__(256) void hyper_norm_kernel(
                 }
             }
 #pragma unroll
-            for (int k = 0; k < HC_MAXS; ++k)
+            for (int k = 0; k < NSTR; ++k)
                 if (k < S) {
 #pragma unroll
                     for (int e = 0; e < W; ++e) x[k][e] = nx[k][e];
@@ -113,7 +115,7 @@ __global__ __launch_bounds__(256) void hyper_norm_kernel(
         for (int e = 0; e < W; ++e) {
             float acc = 0.0f;
 #pragma unroll
-            for (int s = 0; s < HC_MAXS; ++s)
+            for (int s = 0; s < NSTR; ++s)
                 if (s < S) acc = fmaf(srd[s], x[s][e], acc);
             u[e] = acc;
         }
@@ -219,11 +221,20 @@ extern "C" int oa_hyper_norm(void* stream, void* streams, int S, const void* y, 
     };
     const bool vec = C % 4 == 0 && (uintptr_t)streams % 16 == 0 && al(y, ys) && al(y2, y2s) &&
                      al(out, 0);
-#define HC_LAUNCH(TC, V)                                                                          \
-    hipLaunchKernelGGL((hyper_norm_kernel<TC, V>), dim3(T), dim3(256), 0, s, (float*)streams, S,  \
-                       (const TC*)y, ys, (const TC*)y2, y2s, (const float*)g2, g2s,                \
+#define HC_LAUNCH_N(TC, V, N)                                                                     \
+    hipLaunchKernelGGL((hyper_norm_kernel<TC, V, N>), dim3(T), dim3(256), 0, s, (float*)streams,  \
+                       S, (const TC*)y, ys, (const TC*)y2, y2s, (const float*)g2, g2s,             \
                        (const float*)mix, (const float*)write, (const float*)read,                \
                        (const float*)w, (const float*)b, (TC*)out, C, eps)
+    // one to four streams have kernels of their own size; more share the widest
+#define HC_LAUNCH(TC, V)                              \
+    do {                                              \
+        if (S == 1) HC_LAUNCH_N(TC, V, 1);            \
+        else if (S == 2) HC_LAUNCH_N(TC, V, 2);       \
+        else if (S == 3) HC_LAUNCH_N(TC, V, 3);       \
+        else if (S == 4) HC_LAUNCH_N(TC, V, 4);       \
+        else HC_LAUNCH_N(TC, V, HC_MAXS);             \
+    } while (0)
     if (dt == 1) {
         if (vec) HC_LAUNCH(float, true);
         else HC_LAUNCH(float, false);
@@ -232,6 +243,7 @@ extern "C" int oa_hyper_norm(void* stream, void* streams, int S, const void* y, 
         else HC_LAUNCH(bf16s, false);
     }
 #undef HC_LAUNCH
+#undef HC_LAUNCH_N
     HIP_CHECK_LAUNCH();
     return 0;
 }
@@ -470,7 +482,7 @@ extern "C" int oa_moe_pairs_up(void* stream, const void* x, const void* w1, cons
     if (T <= 0) return 0;
     if (top < 1 || E < 1 || I < 1 || K < 1 || (act != 0 && act != 1 && act != 3)) return -100;
     const int vec = (K % 8 == 0 && (uintptr_t)x % 32 == 0 && (uintptr_t)w1 % 32 == 0) ? 1 : 0;
-    dim3 grid(T * top, std::min(CEIL_DIV(I, 4), 64));
+    dim3 grid(T * top, std::min(CEIL_DIV(I, 4), 512));
     hipStream_t s = (hipStream_t)stream;
     if (dt == 1)
         hipLaunchKernelGGL((moe_pairs_up_kernel<float>), grid, dim3(256), 0, s, (const float*)x,

@@ -7,6 +7,7 @@
 //
 //   oa_moe_gateup[_fp8]: act[p, :I] = silu(x[tok] @ gate_e^T) * (x[tok] @ up_e^T)
 //   oa_moe_down[_fp8]:   y[p, :H]  = (act[p] @ w2_e^T) * pair_weight[p]
+//   activation 3 (ungated experts, weights [E, I, K]): act[p, :I] = relu(x[tok] @ up_e^T)^2
 //
 // The caller then out.index_add_(0, token_ids, y) — one scatter per layer.
 // Weights: bf16 [E, 2I|H, K] or fp8 [E, 2I|H, K] + per-row f32 scales.
@@ -89,21 +90,24 @@ __global__ __launch_bounds__(256) void moe_gateup_kernel(
     const int wid = threadIdx.x / WAVE;
     const int wwords = FP8 ? K / 4 : K / 2;
     const uint32_t* xrow = x + (size_t)token_ids[p] * (K / 2);
-    const uint32_t* wbase = w + (size_t)e * 2 * I * wwords;
-    const float* sbase = FP8 ? wscale + (size_t)e * 2 * I : nullptr;
+    const bool gated = actk != 3;          // ungated experts hold I rows, not 2I
+    const uint32_t* wbase = w + (size_t)e * (gated ? 2 : 1) * I * wwords;
+    const float* sbase = FP8 ? wscale + (size_t)e * (gated ? 2 : 1) * I : nullptr;
 
     for (int row = blockIdx.x * 4 + wid; row < I; row += gridDim.x * 4) {
-        float g, u;
+        float g, u = 0.0f;
         if (FP8) {
             g = dot_fp8(wbase + (size_t)row * wwords, xrow, wwords, lane) * sbase[row];
-            u = dot_fp8(wbase + (size_t)(I + row) * wwords, xrow, wwords, lane) *
-                sbase[I + row];
+            if (gated)
+                u = dot_fp8(wbase + (size_t)(I + row) * wwords, xrow, wwords, lane) *
+                    sbase[I + row];
         } else {
             g = dot_bf16(wbase + (size_t)row * wwords, xrow, wwords, lane);
-            u = dot_bf16(wbase + (size_t)(I + row) * wwords, xrow, wwords, lane);
+            if (gated) u = dot_bf16(wbase + (size_t)(I + row) * wwords, xrow, wwords, lane);
         }
         if (lane == 0) {
-            const float a = moe_gate_act(g, u, actk, limit, alpha);
+            const float r = fmaxf(g, 0.0f);
+            const float a = gated ? moe_gate_act(g, u, actk, limit, alpha) : r * r;
             reinterpret_cast<uint16_t*>(act)[(size_t)p * I + row] = f32_to_bf16(a);
         }
     }
@@ -150,7 +154,10 @@ __global__ __launch_bounds__(256) void moe_down_kernel(
 #define EMAJ_MAXP 2048   // pair-list capacity (batch 256 x top-k 8)
 #define EMAJ_GROUP 8     // pairs per weight stream
 
-template <bool FP8, bool GATEUP>
+// MODE 0: down projection (rows of act, scaled by the pair weight); 1: gate
+// and up rows with the gate activation; 2: up rows alone (ungated experts,
+// [E, NROWS, K]) with relu squared.
+template <bool FP8, int MODE>
 __global__ __launch_bounds__(256) void moe_emaj_kernel(
     const uint32_t* __restrict__ x,       // [T, K/2] bf16 (or act [P, I/2])
     const uint32_t* __restrict__ w,       // [E, 2I|H, K] bf16/fp8 words
@@ -160,6 +167,7 @@ __global__ __launch_bounds__(256) void moe_emaj_kernel(
     const float* __restrict__ pair_w,     // [P] (down; ignored for gateup)
     uint32_t* __restrict__ out,           // [P, I] or [P, H] bf16
     int P, int NROWS /* I or H */, int K, int actk, float limit, float alpha) {
+    constexpr bool GATEUP = MODE == 1;
     const int e = blockIdx.y;
     const int lane = threadIdx.x & (WAVE - 1);
     const int wid = threadIdx.x / WAVE;
@@ -199,7 +207,7 @@ __global__ __launch_bounds__(256) void moe_emaj_kernel(
                 accg[c] = accu[c] = 0.0f;
                 int p = plist[g0];  // safe default
                 if (c < m) p = plist[g0 + c];
-                xbase[c] = x + (size_t)(GATEUP ? token_ids[p] : p) * xwords;
+                xbase[c] = x + (size_t)(MODE != 0 ? token_ids[p] : p) * xwords;
             }
             // stream the weight row(s) once; dot against every pair's x row
             for (int i = lane * 4; i < wwords; i += WAVE * 4) {
@@ -261,6 +269,11 @@ __global__ __launch_bounds__(256) void moe_emaj_kernel(
                         const float a = moe_gate_act(g, u, actk, limit, alpha);
                         reinterpret_cast<uint16_t*>(out)[(size_t)p * NROWS + row] =
                             f32_to_bf16(a);
+                    } else if (MODE == 2) {
+                        if (FP8) g *= sbase[row];
+                        const float r = fmaxf(g, 0.0f);
+                        reinterpret_cast<uint16_t*>(out)[(size_t)p * NROWS + row] =
+                            f32_to_bf16(r * r);
                     } else {
                         if (FP8) g *= sbase[row];
                         reinterpret_cast<uint16_t*>(out)[(size_t)p * NROWS + row] =
@@ -279,14 +292,28 @@ extern "C" int oa_moe_gateup_emaj_act(void* stream, const void* x, const void* w
                                       float alpha) {
     if (K % 16 != 0 || P > EMAJ_MAXP) return -100;
     dim3 grid(min(64, CEIL_DIV(I, 4)), E), block(256);
+    if (actk == 3) {
+        if (fp8)
+            hipLaunchKernelGGL((moe_emaj_kernel<true, 2>), grid, block, 0, (hipStream_t)stream,
+                               (const uint32_t*)x, (const uint32_t*)w, (const float*)wscale,
+                               (const int*)expert_ids, (const int*)token_ids,
+                               (const float*)nullptr, (uint32_t*)act, P, I, K, actk, limit, alpha);
+        else
+            hipLaunchKernelGGL((moe_emaj_kernel<false, 2>), grid, block, 0, (hipStream_t)stream,
+                               (const uint32_t*)x, (const uint32_t*)w, (const float*)wscale,
+                               (const int*)expert_ids, (const int*)token_ids,
+                               (const float*)nullptr, (uint32_t*)act, P, I, K, actk, limit, alpha);
+        HIP_CHECK_LAUNCH();
+        return 0;
+    }
     if (fp8)
-        hipLaunchKernelGGL((moe_emaj_kernel<true, true>), grid, block, 0,
+        hipLaunchKernelGGL((moe_emaj_kernel<true, 1>), grid, block, 0,
                            (hipStream_t)stream, (const uint32_t*)x,
                            (const uint32_t*)w, (const float*)wscale,
                            (const int*)expert_ids, (const int*)token_ids,
                            (const float*)nullptr, (uint32_t*)act, P, I, K, actk, limit, alpha);
     else
-        hipLaunchKernelGGL((moe_emaj_kernel<false, true>), grid, block, 0,
+        hipLaunchKernelGGL((moe_emaj_kernel<false, 1>), grid, block, 0,
                            (hipStream_t)stream, (const uint32_t*)x,
                            (const uint32_t*)w, (const float*)wscale,
                            (const int*)expert_ids, (const int*)token_ids,
@@ -310,13 +337,13 @@ extern "C" int oa_moe_down_emaj(void* stream, const void* act, const void* w,
     if (I % 16 != 0 || P > EMAJ_MAXP) return -100;
     dim3 grid(min(64, CEIL_DIV(H, 4)), E), block(256);
     if (fp8)
-        hipLaunchKernelGGL((moe_emaj_kernel<true, false>), grid, block, 0,
+        hipLaunchKernelGGL((moe_emaj_kernel<true, 0>), grid, block, 0,
                            (hipStream_t)stream, (const uint32_t*)act,
                            (const uint32_t*)w, (const float*)wscale,
                            (const int*)expert_ids, (const int*)nullptr,
                            (const float*)pair_w, (uint32_t*)y, P, H, I, 0, 0.0f, 0.0f);
     else
-        hipLaunchKernelGGL((moe_emaj_kernel<false, false>), grid, block, 0,
+        hipLaunchKernelGGL((moe_emaj_kernel<false, 0>), grid, block, 0,
                            (hipStream_t)stream, (const uint32_t*)act,
                            (const uint32_t*)w, (const float*)wscale,
                            (const int*)expert_ids, (const int*)nullptr,

@@ -472,7 +472,9 @@ def test_ungated_experts_paths(mode, sizes):
         mlp.force_path = path
         close(mlp(x.to(eng.device)), want, dtype, path, loose=2.0)
     mlp.force_path = None
-    close(mlp(x[:3].to(eng.device)), want[:3], dtype, "default path", loose=2.0)
+    close(mlp(x[:3].to(eng.device)), want[:3], dtype, "default path, few pairs", loose=2.0)
+    close(mlp(x.to(eng.device)), want, dtype, "default path, many pairs", loose=2.0)
+    close(mlp(x.to(eng.device), decode=True), want, dtype, "default path, decode step", loose=2.0)
 
 
 @pytest.mark.parametrize("mode", MODES[:2])
