@@ -15,7 +15,7 @@ CSRC = os.path.join(
 )
 
 FILES = ["gemv.hip", "attention_prefill.hip", "attention_decode.hip", "fp8_moe.hip",
-         "mixers.hip", "blocks.hip", "prenorm.hip", "recurrent.hip"]
+         "mixers.hip", "blocks.hip", "prenorm.hip", "recurrent.hip", "hyper.hip", "moe_gemv.hip"]
 
 # Known, measured-benign exceptions: kernel name fragment -> max scratch
 # bytes/lane. gemm_fp8_kernel_v2<false> (the deep-K register-staged MX GEMM)

@@ -61,5 +61,6 @@ def test_mixers_library_exports():
               "oa_attn_rope_prepare", "oa_act_mul_rows", "oa_route_topk",
               "oa_moe_pairs_gateup", "oa_moe_pairs_down", "oa_add_layer_norm",
               "oa_latent_kv_prepare", "oa_latent_q_assemble", "oa_decay_scan",
-              "oa_gated_rms_norm"]:
+              "oa_gated_rms_norm", "oa_hyper_norm", "oa_rope_rows", "oa_combine_norm_gate",
+              "oa_act_rows", "oa_moe_pairs_up"]:
         assert hasattr(lib, s), f"missing {s}"
