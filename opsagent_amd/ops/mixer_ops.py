@@ -185,6 +185,10 @@ def attn_qkv_prepare(qkv: torch.Tensor, bias: Optional[torch.Tensor], q_norm_w: 
 _GEOM = {}
 
 
+# value channels per head that one launch of the paged attention kernels takes
+ATTN_MAX_VALUES = 256
+
+
 def attn_geometry(H: int, G: int, D: int, Dv: int, dt: int, max_chunk: int) -> Tuple[int, int]:
     """(query tokens per tile, keys per staged tile) of the attention kernel
     for steps whose longest portion is max_chunk tokens."""
@@ -229,6 +233,18 @@ def attention_paged(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
         return torch_ref.attention_paged(q, k_cache, v_cache, sb.cu, sb.past, sb.block_table,
                                          scale, slopes, gate_logits, window or None, sinks,
                                          softcap or None)
+    if Dv > ATTN_MAX_VALUES:
+        # a lane of the kernels holds at most 4 value channels: wider value
+        # heads run as slices of the value channels with the same scores
+        if Gv != 1:
+            raise ValueError(f"value heads wider than {ATTN_MAX_VALUES} need a single value head")
+        out = torch.empty(T, H, Dv, dtype=q.dtype, device=q.device)
+        for lo in range(0, Dv, ATTN_MAX_VALUES):
+            hi = min(Dv, lo + ATTN_MAX_VALUES)
+            part = attention_paged(q, k_cache, v_cache[..., lo:hi], sb, scale, slopes, gate_logits,
+                                   window, sinks, softcap)
+            out[..., lo:hi] = part.view(T, H, hi - lo)
+        return out.view(T, H * Dv)
     lib, hip = _lib()
     dt = _dt(q)
     TQ, KT = attn_geometry(H, G, D, Dv, dt, sb.max_chunk)

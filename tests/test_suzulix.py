@@ -398,7 +398,9 @@ MIXER_GEOMS = {
     "L": [dict(lat_heads=3, lat_dim=8, lat_vdim=14, kv_rank=18, q_rank=22, rot_dim=6),
           dict(lat_heads=4, lat_dim=16, lat_vdim=16, kv_rank=32, q_rank=16, rot_dim=16),
           dict(lat_heads=1, lat_dim=4, lat_vdim=5, kv_rank=9, q_rank=3, rot_dim=2),
-          dict(lat_heads=2, lat_dim=8, lat_vdim=40, kv_rank=64, q_rank=64, rot_dim=32)],
+          dict(lat_heads=2, lat_dim=8, lat_vdim=40, kv_rank=64, q_rank=64, rot_dim=32),
+          # a latent wider than one launch's value channels: two slices of the values
+          dict(lat_heads=3, lat_dim=8, lat_vdim=12, kv_rank=304, q_rank=16, rot_dim=8)],
     "A": [dict(heads=6, kv_heads=2, dim=12, vdim=10, rot_dims=8),
           dict(heads=4, kv_heads=2, dim=32, vdim=16, rot_dims=32),
           dict(heads=2, kv_heads=2, dim=16, vdim=32, rot_dims=0, softcap=None),
